@@ -1,22 +1,27 @@
 """Ops of hybrid decoders that mix paged softmax attention with recurrent layers whose state is carried per sequence:
 
-* `embed_rows`, `offset_rmsnorm`: an fp32 residual from a 16-bit table; an RMS norm whose weight is stored around
-  an offset (x / rms * (offset + w));
+* `embed_rows`, `offset_rmsnorm`, `norm_add`: an fp32 residual from a 16-bit table; an RMS norm whose weight is
+  stored around an offset (x / rms * (offset + w)); the same norm applied to a sublayer's OUTPUT and added to the
+  residual (x += y / rms(y) * (offset + w)), with the 16-bit copy of the new residual the next GEMM reads;
 * `rope_norm_append`: rotary positions on neighbouring pairs of the first `rot_dims` numbers of each query / key
-  head, an optional unit-RMS norm of every head after the rotation, and the append of keys and values to paged pools;
+  head, an optional unit-RMS norm of every head after the rotation (with optional per-channel weights), an optional
+  position-dependent query temperature, and the append of keys and values to paged pools;
 * `masked_attention`: causal attention over the paged pools whose visible range starts at a chunk border
-  (`chunk`), `window` keys back, or at position 0, with an optional sink (one extra term exp(0) in the softmax
-  denominator that carries no value);
+  (`chunk`), `window` keys back, or at position 0, with an optional sink (one extra term exp(0), or exp(s_h) with a
+  learned s_h per head, in the softmax denominator that carries no value), an optional additive bias that depends on
+  the distance between query and key (`log_bucket_table`) and an optional sigmoid gate per token and head;
 * `causal_conv`: a per-channel causal convolution over time (optional bias and SiLU) whose last taps-1 inputs are
   carried per sequence;
-* `unit_norm_heads`, `scan_coefs`, `state_scan`: the pieces of a linear recurrence S <- a S + k u^T, o = S^T q per
-  head (S is [N, P], fp32, one per sequence and head, stored column-major). With `delta` the written value is
-  u = c (v - S^T k) after
-  the decay (gated delta rule), otherwise u = c v with an optional skip D v on the output (state-space duality form);
+* `unit_norm_heads`, `scan_coefs`, `channel_decay`, `state_scan`: the pieces of a linear recurrence
+  S <- a S + k u^T, o = S^T q per head (S is [N, P], fp32, one per sequence and head, stored column-major). With
+  `delta` the written value is u = c (v - S^T k) after the decay (gated delta rule), otherwise u = c v with an
+  optional skip D v on the output (state-space duality form); the decay a is one number per head or, for gated
+  linear attention, one per key channel (S <- diag(a) S + k v^T, a = sigmoid(z)^(1/tau));
 * `gated_group_norm`: unit-RMS norm over groups of columns, a weight, and a SiLU gate before or after the norm;
 * `glu`: silu(a + bias) * (b + bias) with an optional per-row, per-column-group factor (routing weights of experts
   evaluated side by side, or the sigmoid gate of a shared expert);
-* `moe_route`: softmax over experts, the `top` largest, renormalised and scaled, as a dense [T, E] weight matrix.
+* `moe_route`: softmax over experts (optional logit bias), the `top` largest, renormalised and scaled, as a dense
+  [T, E] weight matrix (with eps = 0 and scale = 1 that is the softmax over the chosen logits alone).
 
 Every function runs the HIP kernels of csrc/kernels/hybrid/ on GPU tensors and a plain fp32 PyTorch form on CPU
 tensors (the plumbing path of GPU-less environments). Positions, angles, scores, softmax, norms, routing, decays,
@@ -75,15 +80,59 @@ def offset_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out32: torch.Te
             out16.stride(0) if out16 is not None else 0, M, C, N.stream_ptr())
 
 
+def norm_add(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor, out16: torch.Tensor | None = None,
+             offset: float = 0.0):
+    """x += y / sqrt(mean(y^2) + eps) * (offset + w) for fp32 rows y, x [T, C] (the norm sits on a sublayer's output,
+    the residual takes the normed value); `out16` (bf16 [T, C]) receives the new residual rounded, for the GEMM that
+    reads it next."""
+    T, C = y.shape
+    if T == 0:
+        return x
+    if not y.is_cuda:
+        x.add_(y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float()))
+        if out16 is not None:
+            out16.copy_(x)
+        return x
+    _f32c(y, "norm_add")
+    _f32c(x, "norm_add")
+    N.kcall("mxh_norm_add", y.data_ptr(), y.stride(0), w.data_ptr(), float(offset), float(eps), x.data_ptr(),
+            x.stride(0), N.ptr(out16), out16.stride(0) if out16 is not None else 0, T, C, N.stream_ptr())
+    return x
+
+
 # ------------------------------------------------------------------------------------------------ attention
+def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
+    """Expands a bucketed distance-bias table rel [B, H] into one row per distance: out [ceil(far) + 1, H] fp32 with
+    out[n] = rel[bucket(n)], bucket(n) = n for n < B/2, else min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(far / (B/2))
+    * (B - B/2))). Every distance >= far lands in the last bucket, so the last row serves all of them
+    (`masked_attention` clamps the distance to the table)."""
+    B = rel.shape[0]
+    half = B // 2
+    if half < 1 or far <= half:
+        raise ValueError("log_bucket_table: at least two rows, and the far distance lies beyond the exact half")
+    idx = []
+    for n in range(int(math.ceil(far)) + 1):
+        if n < half:
+            idx.append(n)
+            continue
+        v = math.log(n / half) / math.log(far / half) * (B - half)
+        if abs(v - round(v)) < 1e-9:  # a whole number up to the rounding of the logarithms
+            v = round(v)
+        idx.append(min(B - 1, half + int(math.floor(v))))
+    return rel.float()[torch.tensor(idx, device=rel.device)].contiguous()
+
+
 def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, positions: torch.Tensor, H: int,
                      G: int, dk: int, dv: int, rot_dims: int, rot_base: float, norm: bool, eps: float,
-                     q_out: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, slots: torch.Tensor):
+                     q_out: torch.Tensor, kc: torch.Tensor | None, vc: torch.Tensor | None, slots: torch.Tensor,
+                     q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, q_temp=None):
     """q_in [T, H*dk], k_in [T, G*dk], v_in [T, G*dv]: fp32 column slices of one projection output. Pair (2i, 2i+1)
     of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with `norm` every query
-    and key head is then divided by its root mean square (eps inside the root). Queries go to q_out [T, H*dk]
-    (fp32 or bf16), keys and values into the paged pools kc [blocks, bs, G*dk] / vc [blocks, bs, G*dv] at flat slot
-    slots[t] (slot < 0: not stored)."""
+    and key head is then divided by its root mean square (eps inside the root) and multiplied by q_weight / k_weight
+    (fp32 [dk], shared by the heads) when given. `q_temp` = (coef, every) multiplies the query at position p by
+    1 + coef * ln(floor((p + 1) / every) + 1). Queries go to q_out [T, H*dk] (fp32 or bf16), keys and values into the
+    paged pools kc [blocks, bs, G*dk] / vc [blocks, bs, G*dv] at flat slot slots[t] (slot < 0: not stored). With
+    k_in = None only the queries are made (a layer that reads another layer's keys and values)."""
     T = q_in.shape[0]
     if T == 0:
         return
@@ -92,7 +141,7 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
     if not q_in.is_cuda:
         pos = positions.float()
 
-        def turn(x, n):
+        def turn(x, n, w=None):
             x = x.float().reshape(T, n, dk).clone()
             if rot_dims:
                 i = torch.arange(rot_dims // 2, dtype=torch.float32)
@@ -103,23 +152,42 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
                 x[..., 1:rot_dims:2] = v * c + u * s
             if norm:
                 x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+                if w is not None:
+                    x = x * w.float()
             return x.reshape(T, n * dk)
-        q_out.copy_(turn(q_in, H))
+        qn = turn(q_in, H, q_weight)
+        if q_temp is not None:
+            coef, every = float(q_temp[0]), int(q_temp[1])
+            qn = qn * (1.0 + coef * torch.log((torch.div(positions + 1, every, rounding_mode="floor") + 1).float()))[:, None]
+        q_out.copy_(qn)
+        if k_in is None:
+            return
         ok = slots >= 0
-        kc.view(-1, G * dk)[slots[ok].long()] = turn(k_in, G)[ok].to(kc.dtype)
+        kc.view(-1, G * dk)[slots[ok].long()] = turn(k_in, G, k_weight)[ok].to(kc.dtype)
         vc.view(-1, G * dv)[slots[ok].long()] = v_in.float()[ok].to(vc.dtype)
         return
+    if (q_weight is not None or k_weight is not None) and not norm:
+        raise ValueError("rope_norm_append: head weights belong to the head norm")
+    if k_in is None:  # queries only: no key / value heads in the grid
+        k_in = v_in = q_in
+        kc = vc = q_out
+        G = 0
+    else:
+        if kc.dtype != vc.dtype or not kc.is_contiguous() or not vc.is_contiguous():
+            raise TypeError("rope_norm_append: contiguous key and value pools of one dtype")
     for t_ in (q_in, k_in, v_in):
         _f32c(t_, "rope_norm_append")
-    if kc.dtype != vc.dtype or not kc.is_contiguous() or not vc.is_contiguous():
-        raise TypeError("rope_norm_append: contiguous key and value pools of one dtype")
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 1)
+    if every < 1:
+        raise ValueError("rope_norm_append: the temperature steps every >= 1 positions")
     N.kcall("mxh_rope_norm_append", q_in.data_ptr(), k_in.data_ptr(), v_in.data_ptr(), q_in.stride(0),
             k_in.stride(0), v_in.stride(0), positions.data_ptr(), H, G, dk, dv, rot_dims, float(rot_base), int(norm),
             float(eps), q_out.data_ptr(), q_out.stride(0), _is16(q_out), kc.data_ptr(), vc.data_ptr(), _is16(kc),
-            slots.data_ptr(), T, N.stream_ptr())
+            slots.data_ptr(), N.ptr(q_weight), N.ptr(k_weight), coef, every, T, N.stream_ptr())
 
 
-def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, sink, out, out_scale):
+def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, sink, out, out_scale, sink_v=None,
+              bias=None, gate=None):
     bs = kc.shape[1]
     nb = -(-ctx // bs)
     k = kc[table[:nb].long()].reshape(nb * bs, G, dk)[:ctx].float()
@@ -132,13 +200,18 @@ def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, s
     j = torch.arange(ctx)[None, :]
     lo = (i // chunk) * chunk if chunk else (i - window + 1).clamp(min=0) if window else torch.zeros_like(i)
     vis = (j <= i) & (j >= lo)
+    if bias is not None:
+        s = s + bias.float()[(i - j).clamp(0, bias.shape[0] - 1)].permute(2, 0, 1)
     s = s.masked_fill(~vis[None], float("-inf"))
     m = s.max(-1, keepdim=True).values
     if sink:
-        m = m.clamp(min=0.0)
+        s0 = sink_v.float()[:, None, None] if sink_v is not None else torch.zeros(H, 1, 1)
+        m = torch.maximum(m, s0)
     e = torch.exp(s - m)
-    den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
+    den = e.sum(-1, keepdim=True) + (torch.exp(s0 - m) if sink else 0.0)
     o = torch.einsum("hnj,jhe->nhe", e / den, v.repeat_interleave(rep, 1))
+    if gate is not None:
+        o = o * torch.sigmoid(gate.float())[:, :, None]
     out.copy_((o.reshape(n, H * dv) * out_scale).to(out.dtype))
 
 
@@ -175,7 +248,8 @@ def _visible_blocks(p0: int, n: int, chunk: int, window: int, heads: int):
     return out
 
 
-def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window, sink, out, out_scale):
+def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window, sink, out, out_scale, sink_v=None,
+                     bias=None, gate=None):
     """A long prompt chunk (rows q [n, H*dk] at positions p0 ..) as library GEMMs: per block of rows, the visible keys
     and values are gathered head-major from the pages, scores = Q K^T (fp32), masked sink softmax, out = P V (fp32)."""
     from .dense import bmm_f32
@@ -191,25 +265,30 @@ def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window
         qh = torch.empty((H, n2, dk), dtype=md, device=dev)
         qr = q[a - p0:]
         N.kcall("mxh_head_transpose", qr.data_ptr(), i16, qr.stride(0), dk, qh.data_ptr(), i16, dk, n2 * dk, n2, H, dk,
-                1.0, st)
+                1.0, None, 0, st)
         sc = bmm_f32(qh.view(G, rep * n2, dk), kh.transpose(1, 2))
         pw = torch.empty((G, rep * n2, nk), dtype=md, device=dev)
         N.kcall("mxh_masked_softmax", sc.data_ptr(), pw.data_ptr(), i16, H * n2, n2, nk, a, key0, float(scale),
-                int(chunk), int(window), int(sink), st)
+                int(chunk), int(window), int(sink), N.ptr(sink_v), N.ptr(bias), bias.shape[0] if bias is not None else 0,
+                H, st)
         o = bmm_f32(pw, vh)
         orow = out[a - p0:]
+        grow = gate[a - p0:] if gate is not None else None
         N.kcall("mxh_head_transpose", o.data_ptr(), 0, dv, n2 * dv, orow.data_ptr(), _is16(out), orow.stride(0), dv, n2,
-                H, dv, float(out_scale), st)
+                H, dv, float(out_scale), N.ptr(grow), grow.stride(0) if grow is not None else 0, st)
 
 
 def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: Ragged, H: int, G: int, dk: int, dv: int,
-                     scale: float, out: torch.Tensor, chunk: int = 0, window: int = 0, sink: bool = False,
-                     out_scale: float = 1.0, workspace=None):
+                     scale: float, out: torch.Tensor, chunk: int = 0, window: int = 0, sink=False,
+                     out_scale: float = 1.0, workspace=None, bias: torch.Tensor | None = None,
+                     gate: torch.Tensor | None = None):
     """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key /
     value head h // (H / G). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
-    max(0, i - window + 1) with `window`, else 0. `sink` adds exp(0) to the softmax denominator. out [T, H*dv]
-    (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32 or bf16
-    operands; scores, softmax and the accumulators are fp32.
+    max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
+    [H] adds exp(sink[h]). `bias` (fp32 [L, H], contiguous) adds bias[min(i - j, L - 1), h] to the scaled score.
+    `gate` (fp32 [T, H], may be a column slice) multiplies head h's output of row t by sigmoid(gate[t, h]). out
+    [T, H*dv] (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32
+    or bf16 operands; scores, softmax and the accumulators are fp32.
 
     On the GPU decode rows and short chunks run the row kernel (one wave per row and head; decode rows split their
     visible keys into partitions merged through `workspace` = (fp32 [rows, 2], fp32 [rows, dv]), rows >= n_dec * H
@@ -221,13 +300,22 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
         return out
     if H % G:
         raise ValueError("masked_attention: heads must be a multiple of kv heads")
+    sink_v = sink if isinstance(sink, torch.Tensor) else None
+    sink = sink_v is not None or bool(sink)
+    if sink_v is not None and (sink_v.dtype != torch.float32 or sink_v.numel() != H or not sink_v.is_contiguous()):
+        raise TypeError("masked_attention: one fp32 sink per query head")
+    if bias is not None and (bias.dtype != torch.float32 or bias.dim() != 2 or bias.shape[1] != H
+                             or not bias.is_contiguous()):
+        raise TypeError("masked_attention: the distance bias is a contiguous fp32 [distances, H] table")
+    if gate is not None and (gate.dtype != torch.float32 or gate.shape != (T, H) or gate.stride(1) != 1):
+        raise TypeError("masked_attention: the gate is fp32 [T, H]")
     nd = rag.n_dec
     if not q.is_cuda:
         if nd:
             lens = rag.dec_lens.tolist()
             for i in range(nd):
                 _attn_ref(q[i:i + 1], kc, vc, rag.dec_bt[i], lens[i], lens[i] - 1, H, G, dk, dv, scale, chunk, window,
-                          sink, out[i:i + 1], out_scale)
+                          sink, out[i:i + 1], out_scale, sink_v, bias, gate[i:i + 1] if gate is not None else None)
         if rag.n_pf:
             cu, ctx = rag.pf_cu.tolist(), rag.pf_ctx.tolist()
             for k in range(rag.n_pf):
@@ -235,13 +323,17 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                 if n:
                     r0 = nd + cu[k]
                     _attn_ref(q[r0:r0 + n], kc, vc, rag.pf_bt[k], ctx[k], ctx[k] - n, H, G, dk, dv, scale, chunk,
-                              window, sink, out[r0:r0 + n], out_scale)
+                              window, sink, out[r0:r0 + n], out_scale, sink_v, bias,
+                              gate[r0:r0 + n] if gate is not None else None)
         return out
     if q.dtype != kc.dtype or kc.dtype != vc.dtype or q.stride(1) != 1 or out.stride(1) != 1:
         raise TypeError("masked_attention: queries and pools share one dtype, rows are contiguous")
     bs = kc.shape[1]
     st = N.stream_ptr()
     common = (H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale))
+    nb = bias.shape[0] if bias is not None else 0
+    ldg = gate.stride(0) if gate is not None else 0
+    extra = (N.ptr(sink_v), N.ptr(bias), nb)  # the gate pointer moves with the rows a launch serves
     mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
         bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
     if nd:
@@ -261,19 +353,21 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             N.kcall("mxh_attention_decode_mfma", q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), rag.dec_lens.data_ptr(), nd, out.data_ptr(),
                     out.stride(0), _is16(out), H, G, dk, dv, float(scale), int(chunk), int(window), int(sink),
-                    float(out_scale), parts, plen if parts > 1 else 0, N.ptr(ml), N.ptr(po), st)
+                    float(out_scale), parts, plen if parts > 1 else 0, N.ptr(ml), N.ptr(po), *extra, N.ptr(gate), ldg,
+                    st)
         else:
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
                     out.data_ptr(), out.stride(0), _is16(out), *common, 0, parts, plen if parts > 1 else 0, N.ptr(ml),
-                    N.ptr(po), st)
+                    N.ptr(po), *extra, N.ptr(gate), ldg, st)
     if rag.n_pf:
         lens = rag.pf_q_host if len(rag.pf_q_host) == rag.n_pf and len(rag.pf_ctx_host) == rag.n_pf else None
 
         def rows_kernel(row_off, n_rows):
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
-                    n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, st)
+                    n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, *extra,
+                    N.ptr(gate), ldg, st)
         mfma = mfma_ok
         big = MFMA_MIN_ROWS if mfma else GEMM_MIN_ROWS
         if lens is None or max(lens) < big or (not mfma and 0 < chunk < GEMM_MIN_ROWS):
@@ -286,13 +380,15 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     rows_kernel(run0, r - run0)
                     run0 = None
                 qk, ok = q[nd + r:nd + r + n], out[nd + r:nd + r + n]
+                gk = gate[nd + r:nd + r + n] if gate is not None else None
                 if mfma:
                     N.kcall("mxh_attention_mfma", qk.data_ptr(), qk.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
                             rag.pf_bt[k].data_ptr(), rag.pf_ctx_host[k] - n, n, ok.data_ptr(), ok.stride(0), _is16(out),
-                            H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale), st)
+                            H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale), *extra,
+                            N.ptr(gk), ldg, st)
                 else:
                     _attn_gemm_chunk(qk, kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv, scale, chunk,
-                                     window, sink, ok, out_scale)
+                                     window, sink, ok, out_scale, sink_v, bias, gk)
             elif n and run0 is None:
                 run0 = r
             r += n
@@ -377,14 +473,34 @@ def scan_coefs(a: torch.Tensor, b: torch.Tensor | None, A_log: torch.Tensor, dt_
             A_log.data_ptr(), dt_bias.data_ptr(), decay.data_ptr(), coef.data_ptr(), T, H, N.stream_ptr())
 
 
-def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, coef: torch.Tensor,
+def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: torch.Tensor):
+    """out = sigmoid(z + bias)^(1 / tau), computed as exp(log_sigmoid(z + bias) / tau): the per-channel decay of gated
+    linear attention. z fp32 [T, C] (column slice allowed), bias fp32 [C], out fp32 [T, C] contiguous."""
+    T, C = z.shape
+    if T == 0:
+        return out
+    if not z.is_cuda:
+        x = z.float() + bias.float() if bias is not None else z.float()
+        out.copy_(torch.exp(F.logsigmoid(x) / tau))
+        return out
+    _f32c(z, "channel_decay")
+    if not out.is_contiguous() or out.dtype != torch.float32 or tau <= 0:
+        raise ValueError("channel_decay: contiguous fp32 output, tau > 0")
+    N.kcall("mxh_channel_decay", z.data_ptr(), z.stride(0), N.ptr(bias), float(1.0 / tau), out.data_ptr(), T, C,
+            N.stream_ptr())
+    return out
+
+
+def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, coef: torch.Tensor | None,
                skip: torch.Tensor | None, state: torch.Tensor, rag: Ragged, out: torch.Tensor, H: int, G: int, Nk: int,
-               P: int, delta: bool):
+               P: int, delta: bool, channel: bool = False, q_scale: float = 1.0):
     """Linear recurrence per sequence and head over the step's rows, in order:
         S <- decay_t S;  u = coef_t (v_t - S^T k_t) if delta else coef_t v_t;  S <- S + k_t u^T;
-        o_t = S^T q_t (+ skip_h v_t)
+        o_t = S^T (q_scale q_t) (+ skip_h v_t)
     k, q fp32 [T, G*Nk] (head h reads group h // (H / G)), v fp32 [T, H*P], decay / coef fp32 [T, H], out fp32
-    [T, H*P]; all may be column slices. state fp32 [slots, H, P, Nk] (a column's Nk numbers are contiguous) is read at
+    [T, H*P]; all may be column slices. With `channel` the decay is fp32 [T, H*Nk], one number per head and key
+    channel (row n of S is multiplied by decay[h, n]: gated linear attention). coef = None means 1.
+    state fp32 [slots, H, P, Nk] (a column's Nk numbers are contiguous) is read at
     the sequence's slot unless its first row is at position 0 (then S starts at zero) and written back after its last
     row."""
     T = k.shape[0]
@@ -398,10 +514,11 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
             S = torch.zeros(H, Nk, P) if (pos[r0] == 0 or slot < 0) else state[slot].transpose(1, 2).clone()
             for t in range(r0, r0 + n):
                 kt = k[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
-                qt = q[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
+                qt = q[t].float().reshape(G, Nk).repeat_interleave(rep, 0) * q_scale
                 vt = v[t].float().reshape(H, P)
-                S = S * decay[t][:, None, None]
-                u = coef[t][:, None] * ((vt - torch.einsum("hnp,hn->hp", S, kt)) if delta else vt)
+                S = S * (decay[t].reshape(H, Nk)[:, :, None] if channel else decay[t][:, None, None])
+                cf = coef[t][:, None] if coef is not None else 1.0
+                u = cf * ((vt - torch.einsum("hnp,hn->hp", S, kt)) if delta else vt)
                 S = S + kt[:, :, None] * u[:, None, :]
                 o = torch.einsum("hnp,hn->hp", S, qt)
                 if skip is not None:
@@ -413,12 +530,14 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
     for t_ in (k, q, v, out):
         _f32c(t_, "state_scan")
     if tuple(state.shape[1:]) != (H, P, Nk) or not state.is_contiguous() or not decay.is_contiguous() \
-            or not coef.is_contiguous() or H % G or Nk > 256:
+            or (coef is not None and not coef.is_contiguous()) or H % G or Nk > 256:
         raise ValueError("state_scan: state is [slots, H, P, N] with N <= 256, decay / coef contiguous [T, H]")
+    if decay.shape[-1] != (H * Nk if channel else H) or (channel and delta):
+        raise ValueError("state_scan: one decay per head, or per head and key channel (not with the delta rule)")
     N.kcall("mxh_state_scan", k.data_ptr(), k.stride(0), q.data_ptr(), q.stride(0), v.data_ptr(), v.stride(0),
-            decay.data_ptr(), coef.data_ptr(), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
+            decay.data_ptr(), N.ptr(coef), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
             rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, out.data_ptr(), out.stride(0), H, G, Nk,
-            P, int(delta), N.stream_ptr())
+            P, int(delta), int(channel), float(q_scale), N.stream_ptr())
     return out
 
 
@@ -474,17 +593,19 @@ def glu(a: torch.Tensor, b: torch.Tensor, bias_a: torch.Tensor | None, bias_b: t
     return out
 
 
-def moe_route(logits: torch.Tensor, top: int, scale: float, weights: torch.Tensor, eps: float = 1e-20):
-    """Router of a mixture of experts: s = softmax(logits) over all E experts, the `top` largest are kept, divided by
-    their sum (+ eps) and multiplied by `scale`. logits fp32 [T, E] (column slice allowed); weights fp32 [T, E]
-    contiguous: the chosen experts' weights, 0 elsewhere. Ties go to the lower expert index."""
+def moe_route(logits: torch.Tensor, top: int, scale: float, weights: torch.Tensor, eps: float = 1e-20,
+              bias: torch.Tensor | None = None):
+    """Router of a mixture of experts: s = softmax(logits + bias) over all E experts, the `top` largest are kept,
+    divided by their sum (+ eps) and multiplied by `scale` (eps = 0, scale = 1: the softmax over the chosen logits
+    alone). logits fp32 [T, E] (column slice allowed), bias fp32 [E]; weights fp32 [T, E] contiguous: the chosen
+    experts' weights, 0 elsewhere. Ties go to the lower expert index."""
     T, E = logits.shape
     if T == 0:
         return weights
     if not 0 < top <= E:
         raise ValueError("moe_route: 1 <= top <= experts")
     if not logits.is_cuda:
-        s = torch.softmax(logits.float(), -1)
+        s = torch.softmax(logits.float() + bias.float() if bias is not None else logits.float(), -1)
         tv, ti = torch.topk(s, top, dim=-1)
         weights.zero_()
         weights.scatter_(1, ti, tv / (tv.sum(-1, keepdim=True) + eps) * scale)
@@ -492,6 +613,6 @@ def moe_route(logits: torch.Tensor, top: int, scale: float, weights: torch.Tenso
     _f32c(logits, "moe_route")
     if E > 1024:
         raise ValueError("moe_route: at most 1024 experts")
-    N.kcall("mxh_moe_route", logits.data_ptr(), logits.stride(0), T, E, top, float(scale), float(eps),
+    N.kcall("mxh_moe_route", logits.data_ptr(), logits.stride(0), N.ptr(bias), T, E, top, float(scale), float(eps),
             weights.data_ptr(), N.stream_ptr())
     return weights
