@@ -1,6 +1,9 @@
 // hybrid_attn.hip: causal softmax attention over paged key / value pools with a visible range that starts at a chunk
 // border, a window's edge or position 0, and an optional sink term in the denominator (ops/hybrid.py
 // masked_attention). Pools are token-major: keys [blocks, bs, G * dk], values [blocks, bs, G * dv], fp32 or bf16.
+// Every kernel also takes an AttnExtra: a learned sink score per head instead of 0, an additive bias looked up by the
+// distance between query and key (table [distances, H], the last row serving every larger distance), and a gate per
+// row and head whose sigmoid multiplies the head's output.
 //
 // attn_rows_kernel: one wave per (query row, query head). Keys are taken 64 at a time, one per lane: the lane forms
 // its key's whole score against the query (held in LDS as fp32, pre-multiplied by the scale), the wave updates the
@@ -21,6 +24,21 @@
 namespace {
 
 constexpr int DVU_MAX = 8;  // value columns per lane: heads of up to 512 numbers
+
+struct AttnExtra {
+    const float* sink_v;  // [H] sink scores (null: 0 where a sink is asked for)
+    const float* bias;    // [nb, H] bias by distance (null: none)
+    int nb;
+    const float* gate;    // pre-sigmoid gate of row r and head h at gate[r * ldg + h] (null: none)
+    int ldg;
+};
+MX_DEV float sink_score(const AttnExtra& ex, int h) { return ex.sink_v ? ex.sink_v[h] : 0.f; }
+MX_DEV float dist_bias(const AttnExtra& ex, int dist, int H, int h) {
+    return ex.bias[(long)min(max(dist, 0), ex.nb - 1) * H + h];
+}
+MX_DEV float gate_factor(const AttnExtra& ex, long row, int h) {
+    return ex.gate ? 1.f / (1.f + expf(-ex.gate[row * ex.ldg + h])) : 1.f;
+}
 
 template <bool B16>
 MX_DEV float ld1(const void* p, long i) {
@@ -109,7 +127,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
                                                        int n_seqs, int row_base, void* out, int ldo, int H, int G,
                                                        int dk, int dv, float scale, int chunk, int window, int sink,
                                                        float out_scale, int row_off, int parts, int part_len,
-                                                       float* part_ml, float* part_o) {
+                                                       float* part_ml, float* part_o, AttnExtra ex) {
     extern __shared__ float lds[];  // [REP][dk] queries, [REP][64] weights, [64] row offsets
     float* qs = lds;
     float* ps = lds + REP * dk;
@@ -134,6 +152,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     const long qrow = (long)(row_base + r) * ldq + (long)h0 * dk;
     for (int e = lane; e < REP * dk; e += 64) qs[e] = ld1<B16>(q, qrow + e) * scale;
     int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
+    const int qpos = pos;
     if (parts > 1) {  // this partition's keys; the sink joins in the merge
         lo += z * part_len;
         pos = min(pos, lo + part_len - 1);
@@ -143,7 +162,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
     float m[REP], l[REP], acc[REP][DVU];
 #pragma unroll
     for (int i = 0; i < REP; ++i) {
-        m[i] = sink ? 0.f : -INFINITY;
+        m[i] = sink ? sink_score(ex, h0 + i) : -INFINITY;
         l[i] = sink ? 1.f : 0.f;
 #pragma unroll
         for (int u = 0; u < DVU; ++u) acc[i][u] = 0.f;
@@ -157,6 +176,10 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         if (ok) {
             tok = (long)table[j / bs] * bs + (j % bs);
             dot_row<B16, REP>(kc, (tok * G + g) * dk, qs, dk, sc);
+            if (ex.bias) {
+#pragma unroll
+                for (int i = 0; i < REP; ++i) sc[i] += dist_bias(ex, qpos - j, H, h0 + i);
+            }
         }
         float alpha[REP], p[REP];
 #pragma unroll
@@ -220,7 +243,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
             }
             continue;
         }
-        const float inv = out_scale / l[i];
+        const float inv = out_scale / l[i] * gate_factor(ex, row_base + r, h);
         const long orow = (long)(row_base + r) * ldo + (long)h * dv;
 #pragma unroll
         for (int u = 0; u < DVU; ++u) {
@@ -303,7 +326,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
                                                               const bf16_t* __restrict__ vc, int bs,
                                                               const int* __restrict__ table, int p0, int n, void* out,
                                                               int ldo, int H, int G, int GW, float scale, int chunk,
-                                                              int window, int sink, float out_scale) {
+                                                              int window, int sink, float out_scale, AttnExtra ex) {
     constexpr int KT = 64;
     constexpr int KSTR = (DK + 8) * 2;  // bytes per key row in LDS (padded)
     constexpr int VSTR = (DV + 8) * 2;  // bytes per value row in LDS (padded)
@@ -341,7 +364,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
     int lo_row[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        mrow[i] = sink ? 0.f : -INFINITY;
+        mrow[i] = sink ? sink_score(ex, hq) * LOG2E_ : -INFINITY;
         lrow[i] = sink ? 1.f : 0.f;
         const int qpos = p0 + row_q0 + 4 * g + i;
         lo_row[i] = chunk > 0 ? (qpos / chunk) * chunk : window > 0 ? max(0, qpos - window + 1) : 0;
@@ -379,6 +402,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
             for (int t = 0; t < 4; ++t) {
                 const int kp = kt0 + 16 * t + col;
                 float v = sacc[t][i] * qs;
+                if (ex.bias) v += dist_bias(ex, qpos - kp, H, hq) * LOG2E_;
                 if (kp > qpos || kp < lo_row[i] || qi >= n) v = -INFINITY;
                 sacc[t][i] = v;
                 mx = fmaxf(mx, v);
@@ -422,7 +446,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
     for (int i = 0; i < 4; ++i) {
         const int qi = row_q0 + 4 * g + i;
         if (qi >= n) continue;
-        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] : 0.f;
+        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] * gate_factor(ex, qi, hq) : 0.f;
 #pragma unroll
         for (int nt = 0; nt < DV / 16; ++nt) {
             const size_t o = (size_t)qi * ldo + (size_t)hq * DV + 16 * nt + col;
@@ -448,7 +472,8 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
                                                               const int* __restrict__ ctx, void* out, int ldo, int H,
                                                               int G, float scale, int chunk, int window, int sink,
                                                               float out_scale, int parts, int part_len,
-                                                              float* __restrict__ part_ml, float* __restrict__ part_o) {
+                                                              float* __restrict__ part_ml, float* __restrict__ part_o,
+                                                              AttnExtra ex) {
     constexpr int KT = 32;  // keys per tile: the wave stages its tiles alone, 64 keys would not fit its registers
     constexpr int VSTR = (DV + 8) * 2, PSTR = (KT + 8) * 2;
     constexpr float LOG2E_ = 1.4426950408889634f, LN2_ = 0.6931471805599453f;
@@ -465,6 +490,9 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
         kv_end = min(kv_end, lo + part_len);
         sink = 0;  // joins in the merge
     }
+    int hrow[4];  // query head of each of the lane's result rows (rows beyond the group repeat its last head)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hrow[i] = kvh * (H / G) + min(4 * g + i, H / G - 1);
     const int* table = bt + (size_t)s * bt_stride;
     const float qs = scale * LOG2E_;
     bf16x8 qf[DK / 32];
@@ -483,7 +511,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
     float mrow[4], lrow[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        mrow[i] = sink ? 0.f : -INFINITY;
+        mrow[i] = sink ? sink_score(ex, hrow[i]) * LOG2E_ : -INFINITY;
         lrow[i] = sink ? 1.f : 0.f;
     }
     // key fragments come straight from the pages (lane (g, col) of tile t: key 16 t + col, dims 32 ks + 8 g .. + 7 are 16
@@ -532,6 +560,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
             for (int t = 0; t < KT / 16; ++t) {
                 const int kp = kt0 + 16 * t + col;
                 float v = sacc[t][i] * qs;
+                if (ex.bias) v += dist_bias(ex, qpos - kp, H, hrow[i]) * LOG2E_;
                 if (kp >= kv_end) v = -INFINITY;
                 sacc[t][i] = v;
                 mx = fmaxf(mx, v);
@@ -582,7 +611,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
             for (int nt = 0; nt < DV / 16; ++nt) part_o[pr * DV + 16 * nt + col] = oacc[nt][i];
             continue;
         }
-        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] : 0.f;
+        const float inv = lrow[i] > 0.f ? out_scale / lrow[i] * gate_factor(ex, s, h) : 0.f;
 #pragma unroll
         for (int nt = 0; nt < DV / 16; ++nt) {
             const size_t o = (size_t)s * ldo + (size_t)h * DV + 16 * nt + col;
@@ -600,17 +629,18 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
 template <bool O16>
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* part_ml, const float* part_o, int parts, int H,
                                                         int dv, int sink, float out_scale, int row_base, void* out,
-                                                        int ldo) {
+                                                        int ldo, AttnExtra ex) {
     constexpr int DVU = DVU_MAX;
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const long p0 = ((long)r * H + h) * parts;
     const int zc = min(lane, parts - 1);
     const float mz = part_ml[(p0 + zc) * 2], lz = lane < parts ? part_ml[(p0 + zc) * 2 + 1] : 0.f;
     float M = wave_max(lz > 0.f ? mz : -INFINITY);
-    if (sink) M = fmaxf(M, 0.f);
+    const float s0 = sink_score(ex, h);
+    if (sink) M = fmaxf(M, s0);
     const float w = lz > 0.f ? expf(mz - M) : 0.f;
-    const float L = wave_sum(lz * w) + (sink ? expf(-M) : 0.f);
-    const float inv = out_scale / L;
+    const float L = wave_sum(lz * w) + (sink ? expf(s0 - M) : 0.f);
+    const float inv = out_scale / L * gate_factor(ex, row_base + r, h);
     const long orow = (long)(row_base + r) * ldo + (long)h * dv;
 #pragma unroll
     for (int u = 0; u < DVU; ++u) {
@@ -652,8 +682,9 @@ __global__ __launch_bounds__(64) void kv_gather_kernel(const E* kc, const E* vc,
 // grid (n, H): dst[i * d_si + h * d_sh + e] = scale * src[i * s_si + h * s_sh + e], e < d
 template <bool S16, bool D16>
 __global__ __launch_bounds__(64) void head_transpose_kernel(const void* src, long s_si, long s_sh, void* dst, long d_si,
-                                                            long d_sh, int d, float scale) {
+                                                            long d_sh, int d, float scale, const float* gate, int ldg) {
     const long so = blockIdx.x * s_si + blockIdx.y * s_sh, dof = blockIdx.x * d_si + blockIdx.y * d_sh;
+    if (gate) scale /= 1.f + expf(-gate[(long)blockIdx.x * ldg + blockIdx.y]);  // sigmoid gate of (row, head)
     for (int e = threadIdx.x; e < d; e += 64) {
         const float v = ld1<S16>(src, so + e) * scale;
         if constexpr (D16) ((bf16_t*)dst)[dof + e] = f32_to_bf16(v);
@@ -665,23 +696,27 @@ __global__ __launch_bounds__(64) void head_transpose_kernel(const void* src, lon
 // key0 .. key0 + nk - 1. Writes the masked, sink-normalised softmax weights (zeros outside the visible range).
 template <bool P16>
 __global__ __launch_bounds__(256) void masked_softmax_kernel(const float* sc, void* pw, int n, int nk, int p0, int key0,
-                                                             float scale, int chunk, int window, int sink) {
+                                                             float scale, int chunk, int window, int sink,
+                                                             const float* sink_v, const float* bias, int nb, int H) {
     __shared__ float red[4];
     const long row = blockIdx.x;
-    const int i = (int)(row % n);
+    const int i = (int)(row % n), h = (int)(row / n);
     const int pos = p0 + i;
     const int lo = chunk > 0 ? (pos / chunk) * chunk : window > 0 ? max(0, pos - window + 1) : 0;
     const int a = max(lo, key0) - key0, b = min(pos - key0, nk - 1);  // visible local range [a, b]
     const float* s = sc + row * nk;
-    float m = sink ? 0.f : -INFINITY;
-    for (int j = a + threadIdx.x; j <= b; j += 256) m = fmaxf(m, s[j] * scale);
+    const float s0 = sink_v ? sink_v[h] : 0.f;
+    const int d0 = pos - key0;  // distance of local key j: d0 - j
+    auto score = [&](int j) { return s[j] * scale + (bias ? bias[(long)min(d0 - j, nb - 1) * H + h] : 0.f); };
+    float m = sink ? s0 : -INFINITY;
+    for (int j = a + threadIdx.x; j <= b; j += 256) m = fmaxf(m, score(j));
     m = block_max<256>(m, red);
     float l = 0.f;
-    for (int j = a + threadIdx.x; j <= b; j += 256) l += expf(s[j] * scale - m);
-    l = block_sum<256>(l, red) + (sink ? expf(-m) : 0.f);
+    for (int j = a + threadIdx.x; j <= b; j += 256) l += expf(score(j) - m);
+    l = block_sum<256>(l, red) + (sink ? expf(s0 - m) : 0.f);
     const float inv = 1.f / l;
     for (int j = threadIdx.x; j < nk; j += 256) {
-        const float p = (j >= a && j <= b) ? expf(s[j] * scale - m) * inv : 0.f;
+        const float p = (j >= a && j <= b) ? expf(score(j) - m) * inv : 0.f;
         if constexpr (P16) ((bf16_t*)pw)[row * nk + j] = f32_to_bf16(p);
         else ((float*)pw)[row * nk + j] = p;
     }
@@ -696,8 +731,11 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
                              int bt_stride, const int* cu_q, const int* ctx, int n_seqs, int n_rows, int row_base,
                              void* out, int ldo, int o16, int H, int G, int dk, int dv, float scale, int chunk,
                              int window, int sink, float out_scale, int row_off, int parts, int part_len,
-                             float* part_ml, float* part_o, hipStream_t st) {
+                             float* part_ml, float* part_o, const float* sink_v, const float* bias, int nb,
+                             const float* gate, int ldg, hipStream_t st) {
     if (n_rows <= 0 || n_seqs <= 0) return 0;
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0);
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU_MAX && dk <= 4096);
     MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535 && row_off >= 0);
@@ -712,7 +750,7 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
 #define GO3(B, O, R, D)                                                                                               \
     attn_rows_kernel<B, O, R, D><<<grid, 64, sh, st>>>(q, ldq, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, row_base, \
                                                        out, ldo, H, G, dk, dv, scale, chunk, window, sink, out_scale, \
-                                                       row_off, parts, part_len, part_ml, part_o)
+                                                       row_off, parts, part_len, part_ml, part_o, ex)
 #define GO(B, O)                                  \
     do {                                          \
         if (dv <= 128) GO3(B, O, REP, 2);         \
@@ -726,8 +764,8 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
 #undef GO3
     if (parts > 1) {
         const dim3 g2(n_rows, H);
-        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo);
-        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo);
+        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo, ex);
+        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, row_base, out, ldo, ex);
     }
     return (int)hipGetLastError();
 }
@@ -745,11 +783,12 @@ extern "C" int mxh_kv_gather(const void* kc, const void* vc, int is16, int bs, c
 }
 
 extern "C" int mxh_head_transpose(const void* src, int s16, long s_si, long s_sh, void* dst, int d16, long d_si,
-                                  long d_sh, int n, int H, int d, float scale, hipStream_t st) {
+                                  long d_sh, int n, int H, int d, float scale, const float* gate, int ldg,
+                                  hipStream_t st) {
     if (n <= 0) return 0;
-    MXH_CHECK(src && dst && H > 0 && H <= 65535 && d > 0);
+    MXH_CHECK(src && dst && H > 0 && H <= 65535 && d > 0 && (!gate || ldg >= H));
     const dim3 grid(n, H);
-#define GO(S, D) head_transpose_kernel<S, D><<<grid, 64, 0, st>>>(src, s_si, s_sh, dst, d_si, d_sh, d, scale)
+#define GO(S, D) head_transpose_kernel<S, D><<<grid, 64, 0, st>>>(src, s_si, s_sh, dst, d_si, d_sh, d, scale, gate, ldg)
     if (s16 && d16) GO(true, true);
     else if (s16) GO(true, false);
     else if (d16) GO(false, true);
@@ -759,11 +798,17 @@ extern "C" int mxh_head_transpose(const void* src, int s16, long s_si, long s_sh
 }
 
 extern "C" int mxh_masked_softmax(const float* sc, void* pw, int p16, long rows, int n, int nk, int p0, int key0,
-                                  float scale, int chunk, int window, int sink, hipStream_t st) {
+                                  float scale, int chunk, int window, int sink, const float* sink_v,
+                                  const float* bias, int nb, int H, hipStream_t st) {
     if (rows <= 0) return 0;
     MXH_CHECK(sc && pw && n > 0 && nk > 0 && rows % n == 0 && rows < (1L << 31) && key0 >= 0 && p0 >= key0);
-    if (p16) masked_softmax_kernel<true><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
-    else masked_softmax_kernel<false><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink);
+    MXH_CHECK((!bias || nb > 0) && (!(bias || sink_v) || rows == (long)H * n));
+    if (p16)
+        masked_softmax_kernel<true><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink,
+                                                                    sink_v, bias, nb, H);
+    else
+        masked_softmax_kernel<false><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink,
+                                                                     sink_v, bias, nb, H);
     return (int)hipGetLastError();
 }
 
@@ -773,8 +818,11 @@ extern "C" int mxh_attention_mfma_ok(int dk, int dv) { return (dk == 64 || dk ==
 
 extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const void* vc, int bs, const int* table,
                                   int p0, int n, void* out, int ldo, int o16, int H, int G, int dk, int dv,
-                                  float scale, int chunk, int window, int sink, float out_scale, hipStream_t st) {
+                                  float scale, int chunk, int window, int sink, float out_scale, const float* sink_v,
+                                  const float* bias, int nb, const float* gate, int ldg, hipStream_t st) {
     if (n <= 0) return 0;
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
     MXH_CHECK(q && kc && vc && table && out && bs > 0 && p0 >= 0 && H > 0 && G > 0 && H % G == 0);
     MXH_CHECK(mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv && chunk >= 0 && window >= 0);
     const int rep = H / G;
@@ -787,11 +835,11 @@ extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const 
         if (o16)                                                                                                      \
             attn_chunk_mfma_kernel<K_, V_, true><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,       \
                                                                        (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
-                                                                       H, G, GW, scale, chunk, window, sink, out_scale); \
+                                                                       H, G, GW, scale, chunk, window, sink, out_scale, ex); \
         else                                                                                                          \
             attn_chunk_mfma_kernel<K_, V_, false><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,      \
                                                                         (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
-                                                                        H, G, GW, scale, chunk, window, sink, out_scale); \
+                                                                        H, G, GW, scale, chunk, window, sink, out_scale, ex); \
     } while (0)
     if (dk == 64 && dv == 64) GO(64, 64);
     else if (dk == 64 && dv == 128) GO(64, 128);
@@ -807,8 +855,11 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
                                          int bt_stride, const int* ctx, int n_seqs, void* out, int ldo, int o16, int H,
                                          int G, int dk, int dv, float scale, int chunk, int window, int sink,
                                          float out_scale, int parts, int part_len, float* part_ml, float* part_o,
+                                         const float* sink_v, const float* bias, int nb, const float* gate, int ldg,
                                          hipStream_t st) {
     if (n_seqs <= 0) return 0;
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0 && H > 0 && G > 0 && H % G == 0);
     MXH_CHECK(H / G <= 16 && G <= 65535 && mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv);
     MXH_CHECK(parts >= 1 && parts <= 64 && (parts == 1 || (part_len > 0 && part_ml && part_o)) && chunk >= 0 && window >= 0);
@@ -818,11 +869,11 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
         if (o16)                                                                                                         \
             attn_decode_mfma_kernel<K_, V_, true><<<grid, 64, 0, st>>>(                                                  \
                 (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
-                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o);                                       \
+                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o, ex);                                       \
         else                                                                                                             \
             attn_decode_mfma_kernel<K_, V_, false><<<grid, 64, 0, st>>>(                                                 \
                 (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
-                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o);                                       \
+                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o, ex);                                       \
     } while (0)
     if (dk == 64 && dv == 64) GO(64, 64);
     else if (dk == 64 && dv == 128) GO(64, 128);
@@ -831,8 +882,8 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
 #undef GO
     if (parts > 1) {
         const dim3 g2(n_seqs, H);
-        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo);
-        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo);
+        if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo, ex);
+        else attn_merge_kernel<false><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo, ex);
     }
     return (int)hipGetLastError();
 }

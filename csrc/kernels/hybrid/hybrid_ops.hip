@@ -1,6 +1,7 @@
 // hybrid_ops.hip: the fp32 row kernels of hybrid attention / recurrent decoders (ops/hybrid.py): embedding gather,
-// offset RMS norm, rotary + head norm + paged append, causal convolution with carried tails, unit-length heads,
-// decay / write-strength coefficients, gated group norm, gated linear unit with per-group factors, expert routing.
+// offset RMS norm, output norm + residual add, rotary + head norm (+ weights, query temperature) + paged append, causal
+// convolution with carried tails, unit-length heads, decay / write-strength coefficients, per-channel decays, gated
+// group norm, gated linear unit with per-group factors, expert routing.
 //
 // All statistics, angles, gates, routing and the residual are fp32; 16-bit (bf16) appears only on outputs that feed a
 // GEMM and in the paged pools. Launchers are `extern "C" int mxh_*(..., hipStream_t)`, return the launch's
@@ -99,6 +100,54 @@ __global__ __launch_bounds__(NT) void offset_norm_kernel(const float* x, int ldx
     }
 }
 
+// x[t] += y[t] / rms(y[t]) * (offset + w); o16 (optional) = the new x[t] rounded. One block per row, the row of y kept
+// in registers when it fits.
+__global__ __launch_bounds__(NT) void norm_add_kernel(const float* y, int ldy, const float* w, float offset, float eps,
+                                                      float* x, int ldx, bf16_t* o16, int ld16, int C) {
+    __shared__ float red[NT / 64];
+    const int i = blockIdx.x;
+    const float* yr = y + (long)i * ldy;
+    float* xr = x + (long)i * ldx;
+    const bool cached = C <= NT * RC;
+    float keep[RC], wk[RC], xk[RC];
+    float ss = 0.f;
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
+            const int c = min((int)threadIdx.x + k * NT, C - 1);
+            const float v = yr[c];
+            wk[k] = w[c];
+            xk[k] = xr[c];
+            keep[k] = (int)threadIdx.x + k * NT < C ? v : 0.f;
+            ss += keep[k] * keep[k];
+        }
+    } else {
+        for (int c = threadIdx.x; c < C; c += NT) {
+            const float v = yr[c];
+            ss += v * v;
+        }
+    }
+    ss = block_sum_dyn(ss, red);
+    const float sc = 1.f / sqrtf(ss / (float)C + eps);
+    if (cached) {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+            const int c = threadIdx.x + k * NT;
+            if (c < C) {
+                const float v = xk[k] + keep[k] * sc * (offset + wk[k]);
+                xr[c] = v;
+                if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
+            }
+        }
+        return;
+    }
+    for (int c = threadIdx.x; c < C; c += NT) {
+        const float v = xr[c] + yr[c] * sc * (offset + w[c]);
+        xr[c] = v;
+        if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
+    }
+}
+
 // grid (T, H + 2G), one wave per (token, head): query heads, then key heads, then value heads. Element e < rot_dims
 // of a query / key head turns with its neighbour e ^ 1 by angle pos * base^(-(e / 2) * 2 / rot_dims).
 constexpr int HEAD_E = 8;  // elements per lane: heads of up to 512 numbers
@@ -107,7 +156,8 @@ __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, c
                                                               int ldq, int ldk, int ldv, const int* positions, int H,
                                                               int G, int dk, int dv, int rot, float neg_log_base,
                                                               int norm, float eps, void* qo, int ldqo, void* kc,
-                                                              void* vc, const int* slots) {
+                                                              void* vc, const int* slots, const float* qw,
+                                                              const float* kw, float temp_coef, int temp_every) {
     const int t = blockIdx.x, u = blockIdx.y, lane = threadIdx.x;
     if (u >= H + G) {  // value head: plain copy into the pool
         const int sl = slots[t];
@@ -148,13 +198,17 @@ __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, c
     }
     float sc = 1.f;
     if (norm) sc = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+    // the head norm's weight (shared by the heads) and, for queries, the temperature of the position
+    const float* hw = isq ? qw : kw;
+    if (isq && temp_coef != 0.f) sc *= 1.f + temp_coef * logf((float)((positions[t] + 1) / temp_every + 1));
     const long dst = isq ? (long)t * ldqo + (long)hd * dk : ((long)sl * G + hd) * dk;
 #pragma unroll
     for (int k = 0; k < HEAD_E; ++k) {
         const int e = lane + k * 64;
         if (e < dk) {
-            if (isq) st_elem<Q16>(qo, dst + e, val[k] * sc);
-            else st_elem<C16>(kc, dst + e, val[k] * sc);
+            const float v = hw ? val[k] * sc * hw[e] : val[k] * sc;
+            if (isq) st_elem<Q16>(qo, dst + e, v);
+            else st_elem<C16>(kc, dst + e, v);
         }
     }
 }
@@ -253,6 +307,15 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
     coef[i] = b ? sigmoid_acc(b[(long)t * ldb + h]) : s;
 }
 
+// out = exp(log_sigmoid(z + bias) * inv_tau) = sigmoid(z + bias)^(1 / tau)
+__global__ __launch_bounds__(NT) void channel_decay_kernel(const float* z, int ldz, const float* bias, float inv_tau,
+                                                           float* out, int C) {
+    const int c = blockIdx.y * NT + threadIdx.x, t = blockIdx.x;
+    if (c >= C) return;
+    const float x = z[(long)t * ldz + c] + (bias ? bias[c] : 0.f);
+    out[(long)t * C + c] = expf(-softplus_acc(-x) * inv_tau);
+}
+
 // grid (T, C / group): one block per (token, group of columns). Groups of up to blockDim * GC numbers are read once
 // (straight-line clamped loads, all in flight together) and kept in registers with their gates; the launcher picks
 // the smallest GC that holds the group
@@ -334,8 +397,8 @@ __global__ __launch_bounds__(NT) void glu_kernel(const float* a, int lda, const 
 
 // one wave per token; lane l holds experts l, l + 64, ... (up to 16 each)
 constexpr int ROUTE_E = 16;
-__global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int ld, int E, int top, float scale,
-                                                       float eps, float* weights) {
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int ld, const float* bias, int E, int top,
+                                                       float scale, float eps, float* weights) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (long)t * ld;
     float v[ROUTE_E];
@@ -343,7 +406,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int 
 #pragma unroll
     for (int k = 0; k < ROUTE_E; ++k) {
         const int e = lane + k * 64;
-        v[k] = e < E ? z[e] : -INFINITY;
+        v[k] = e < E ? z[e] + (bias ? bias[e] : 0.f) : -INFINITY;
         m = fmaxf(m, v[k]);
     }
     m = wave_max(m);
@@ -418,19 +481,29 @@ extern "C" int mxh_offset_norm(const float* x, int ldx, const int* rows, const f
     return (int)hipGetLastError();
 }
 
+extern "C" int mxh_norm_add(const float* y, int ldy, const float* w, float offset, float eps, float* x, int ldx,
+                            bf16_t* o16, int ld16, int T, int C, hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(y && w && x && C > 0 && ldy >= C && ldx >= C && (!o16 || ld16 >= C));
+    norm_add_kernel<<<T, NT, 0, st>>>(y, ldy, w, offset, eps, x, ldx, o16, ld16, C);
+    return (int)hipGetLastError();
+}
+
 extern "C" int mxh_rope_norm_append(const float* qi, const float* ki, const float* vi, int ldq, int ldk, int ldv,
                                     const int* positions, int H, int G, int dk, int dv, int rot, float base, int norm,
                                     float eps, void* qo, int ldqo, int q16, void* kc, void* vc, int c16,
-                                    const int* slots, int T, hipStream_t st) {
+                                    const int* slots, const float* qw, const float* kw, float temp_coef,
+                                    int temp_every, int T, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(qi && ki && vi && positions && qo && kc && vc && slots);
-    MXH_CHECK(H > 0 && G > 0 && dk > 0 && dv > 0 && dk <= 64 * HEAD_E && rot >= 0 && rot <= dk && rot % 2 == 0);
+    MXH_CHECK(qi && ki && vi && positions && qo && kc && vc && slots && temp_every >= 1);
+    // G == 0: queries only (keys and values of another layer are read)
+    MXH_CHECK(H > 0 && G >= 0 && dk > 0 && dv > 0 && dk <= 64 * HEAD_E && rot >= 0 && rot <= dk && rot % 2 == 0);
     MXH_CHECK(ldq >= H * dk && ldk >= G * dk && ldv >= G * dv && ldqo >= H * dk && base > 0.f);
     const dim3 grid(T, H + 2 * G);
     const float nlb = -logf(base);
 #define GO(Q, C)                                                                                                   \
     rope_norm_append_kernel<Q, C><<<grid, 64, 0, st>>>(qi, ki, vi, ldq, ldk, ldv, positions, H, G, dk, dv, rot, nlb, \
-                                                       norm, eps, qo, ldqo, kc, vc, slots)
+                                                       norm, eps, qo, ldqo, kc, vc, slots, qw, kw, temp_coef, temp_every)
     if (q16 && c16) GO(true, true);
     else if (q16) GO(true, false);
     else if (c16) GO(false, true);
@@ -472,6 +545,14 @@ extern "C" int mxh_scan_coefs(const float* a, int lda, const float* b, int ldb, 
     return (int)hipGetLastError();
 }
 
+extern "C" int mxh_channel_decay(const float* z, int ldz, const float* bias, float inv_tau, float* out, int T, int C,
+                                 hipStream_t st) {
+    if (T <= 0) return 0;
+    MXH_CHECK(z && out && C > 0 && ldz >= C && inv_tau > 0.f && C <= 65535 * NT);
+    channel_decay_kernel<<<dim3(T, (C + NT - 1) / NT), NT, 0, st>>>(z, ldz, bias, inv_tau, out, C);
+    return (int)hipGetLastError();
+}
+
 extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
                                     float eps, int group, int gate_first, float out_scale, void* out, int ldo,
                                     int o16, int T, int C, hipStream_t st) {
@@ -507,10 +588,10 @@ extern "C" int mxh_glu(const float* a, int lda, const float* b, int ldb, const f
     return (int)hipGetLastError();
 }
 
-extern "C" int mxh_moe_route(const float* logits, int ld, int T, int E, int top, float scale, float eps,
-                             float* weights, hipStream_t st) {
+extern "C" int mxh_moe_route(const float* logits, int ld, const float* bias, int T, int E, int top, float scale,
+                             float eps, float* weights, hipStream_t st) {
     if (T <= 0) return 0;
     MXH_CHECK(logits && weights && E > 0 && E <= 64 * ROUTE_E && top > 0 && top <= E && ld >= E);
-    moe_route_kernel<<<T, 64, 0, st>>>(logits, ld, E, top, scale, eps, weights);
+    moe_route_kernel<<<T, 64, 0, st>>>(logits, ld, bias, E, top, scale, eps, weights);
     return (int)hipGetLastError();
 }

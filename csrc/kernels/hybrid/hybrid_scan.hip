@@ -11,6 +11,8 @@
 // registers meanwhile, so memory latency and the barrier are paid once per 8 or 16 steps. The state is read from the
 // sequence's slot unless the chunk starts at position 0, and written back after the chunk's last row: a decode row is
 // a chunk of one, a prompt chunk walks its rows inside one launch.
+// CHD (gated linear attention): the decay is one number per head and state row, a_t[n], staged beside k_t and q_t:
+// S[n][p] <- a_t[n] S[n][p] + k_t[n] u[p]. A missing write strength means 1; q_t is multiplied by q_scale when staged.
 #include "../mx_common.h"
 
 namespace {
@@ -32,19 +34,20 @@ MX_DEV float lanes_sum(float v) {
 }
 
 // grid (column blocks, H, sequences); block = 256 threads = 256 / LPC columns
-template <int NPL, int LPC, bool DELTA>
+template <int NPL, int LPC, bool DELTA, bool CHD>
 __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk, const float* q, int ldq,
                                                          const float* v, int ldv, const float* decay, const float* coef,
                                                          const float* skip, float* state, const int* seq_state,
                                                          const int* positions, int n_dec, const int* pf_cu, float* out,
-                                                         int ldo, int H, int G, int N, int P) {
+                                                         int ldo, int H, int G, int N, int P, float q_scale) {
     static_assert(LPC == 4 || LPC == 16, "a column's lanes are a quad or a DPP row");
     constexpr int NT = 256;
     constexpr int NP = NPL * LPC;  // padded N
     constexpr int COLS = NT / LPC;
     constexpr int TB = NP <= 128 ? 16 : 8;  // tokens staged together
-    constexpr int KQ_PT = TB * 2 * NP / NT, V_PT = (TB * COLS + NT - 1) / NT;
-    __shared__ float kq[2][TB][2][NP];
+    constexpr int NW = CHD ? 3 : 2;  // vectors of N numbers staged per token: k, q (, channel decays)
+    constexpr int KQ_PT = TB * NW * NP / NT, V_PT = (TB * COLS + NT - 1) / NT;
+    __shared__ float kq[2][TB][NW][NP];
     __shared__ float vs[2][TB][COLS];
     __shared__ float ac[2][TB][2];
     const int cl = threadIdx.x / LPC;
@@ -100,9 +103,12 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
 #pragma unroll
         for (int i = 0; i < KQ_PT; ++i) {
             const int idx = threadIdx.x + i * NT;
-            const int tt = idx / (2 * NP), w = (idx / NP) & 1, e = idx % NP;
+            const int tt = idx / (NW * NP), w = (idx / NP) % NW, e = idx % NP;
             const long row = min(r0 + tt, last);
-            const float x = w ? qp[row * ldq + min(e, N - 1)] : kp[row * ldk + min(e, N - 1)];
+            const int ec = min(e, N - 1);
+            float x;
+            if (CHD && w == 2) x = decay[row * ((long)H * N) + (long)h * N + ec];
+            else x = w ? qp[row * ldq + ec] * q_scale : kp[row * ldk + ec];
             st_kq[i] = e < N ? x : 0.f;
         }
 #pragma unroll
@@ -114,7 +120,8 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
         }
         if (threadIdx.x < 2 * TB) {
             const long row = min(r0 + (int)threadIdx.x / 2, last);
-            st_ac = (threadIdx.x & 1) ? coef[row * H + h] : decay[row * H + h];
+            if (threadIdx.x & 1) st_ac = coef ? coef[row * H + h] : 1.f;
+            else st_ac = CHD ? 1.f : decay[row * H + h];
         }
     };
     auto publish = [&](int b) {
@@ -150,6 +157,11 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
                     d1 += S[j + 1] * kb[j + 1];
                 }
                 u = cf * (vv - lanes_sum<LPC>(d0 + d1));
+            } else if constexpr (CHD) {
+                const float* ab = &kq[b][tt][NW - 1][part * NPL];
+#pragma unroll
+                for (int j = 0; j < NPL; ++j) S[j] *= ab[j];
+                u = cf * vv;
             } else {
 #pragma unroll
                 for (int j = 0; j < NPL; ++j) S[j] *= a;
@@ -191,26 +203,27 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
 extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, const float* v, int ldv,
                               const float* decay, const float* coef, const float* skip, float* state,
                               const int* seq_state, const int* positions, int n_dec, const int* pf_cu, int n_pf,
-                              float* out, int ldo, int H, int G, int N, int P, int delta, hipStream_t st) {
+                              float* out, int ldo, int H, int G, int N, int P, int delta, int channel, float q_scale,
+                              hipStream_t st) {
     const int n_seqs = n_dec + n_pf;
     if (n_seqs <= 0) return 0;
-    MXH_CHECK(k && q && v && decay && coef && state && seq_state && positions && out && (n_pf == 0 || pf_cu));
+    MXH_CHECK(k && q && v && decay && state && seq_state && positions && out && (n_pf == 0 || pf_cu));
+    MXH_CHECK(!(delta && channel));
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && N > 0 && N <= 256 && P > 0 && H <= 65535 && n_seqs <= 65535);
     MXH_CHECK(ldk >= G * N && ldq >= G * N && ldv >= H * P && ldo >= H * P);
     const int lpc = N <= 32 ? 4 : 16;
     const int threads = 256;
     const int cols = threads / lpc;
     const dim3 grid((P + cols - 1) / cols, H, n_seqs);
-#define GO(NPL, LPC)                                                                                                 \
-    do {                                                                                                             \
-        if (delta)                                                                                                   \
-            state_scan_kernel<NPL, LPC, true><<<grid, threads, 0, st>>>(k, ldk, q, ldq, v, ldv, decay, coef, skip,   \
-                                                                        state, seq_state, positions, n_dec, pf_cu,  \
-                                                                        out, ldo, H, G, N, P);                       \
-        else                                                                                                         \
-            state_scan_kernel<NPL, LPC, false><<<grid, threads, 0, st>>>(k, ldk, q, ldq, v, ldv, decay, coef, skip,  \
-                                                                         state, seq_state, positions, n_dec, pf_cu, \
-                                                                         out, ldo, H, G, N, P);                      \
+#define GO2(NPL, LPC, D_, C_)                                                                                      \
+    state_scan_kernel<NPL, LPC, D_, C_><<<grid, threads, 0, st>>>(k, ldk, q, ldq, v, ldv, decay, coef, skip, state,    \
+                                                                  seq_state, positions, n_dec, pf_cu, out, ldo, H, G, \
+                                                                  N, P, q_scale)
+#define GO(NPL, LPC)                              \
+    do {                                          \
+        if (delta) GO2(NPL, LPC, true, false);    \
+        else if (channel) GO2(NPL, LPC, false, true); \
+        else GO2(NPL, LPC, false, false);         \
     } while (0)
     if (N <= 16) GO(4, 4);
     else if (N <= 32) GO(8, 4);
@@ -218,5 +231,6 @@ extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, 
     else if (N <= 128) GO(8, 16);
     else GO(16, 16);
 #undef GO
+#undef GO2
     return (int)hipGetLastError();
 }
