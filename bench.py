@@ -96,12 +96,13 @@ def parse():
                     help="comma list of sampling phases measured back to back on the same server: reference = "
                          "the reference's defaults (temperature 0.9, top_k 40, top_p 0.95; backend_config.go "
                          "SetDefaults) on the GPU sampler; greedy = argmax. The first phase is the headline")
-    ap.add_argument("--arch-bench", default="", choices=["", "vosotar", "vugotar"],
+    ap.add_argument("--arch-bench", default="", choices=["", "vosotar", "vugotar", "girulorn"],
                     help="instead of the headline serving benchmark: prefill and decode throughput of this model "
                          "family beside the Llama graph at equal layer sizes (random bf16 / f16 weights, one GPU)")
     ap.add_argument("--arch-sizes", default="1b,7b", help="--arch-bench: comma list of layer sizes (1b, 7b)")
     ap.add_argument("--arch-layers", type=int, default=4, help="--arch-bench: layers per model")
-    ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, vugotar, llama-f16)")
+    ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, vugotar, girulorn, "
+                         "vugotar-moe, llama-f16)")
     ap.add_argument("--arch-batches", default="1,32", help="--arch-bench: decode batch sizes")
     ap.add_argument("--arch-chunk", type=int, default=2048, help="--arch-bench vugotar: attention chunk size")
     return ap.parse_args()
@@ -234,7 +235,31 @@ def run_arch_bench(args) -> int:
 
     def models(sz):
         s = ARCH_SIZES[sz]
-        if args.arch_bench == "vugotar":
+        if args.arch_bench == "girulorn":
+            # attention and gated-linear-attention layers in turn, every second attention layer reading the keys and
+            # values of the one before it; attention heads as the Llama graph's (GQA 4:1, head size 128), half as many
+            # recurrent heads with 128 x 128 states; 8 experts of a quarter of the feed-forward width, two chosen, and
+            # a shared expert of half of it (as many active feed-forward numbers per token as the dense models). The
+            # closest model of the framework, Vugotar (attention beside a delta rule, a state-space layer every
+            # fourth), runs beside it with the same expert feed-forwards.
+            from localai_tfp_amd.models import girulorn as GI
+            from localai_tfp_amd.models import vugotar as VU
+            pat = tuple("gla" if i % 2 else "attention" for i in range(nl))
+            moe = dict(experts=8, top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 2)
+            gc = GI.make_config(hidden=s["hidden"], vocab=V, pattern=pat, heads=s["heads"],
+                                kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, bias_max=4096.0, bias_rows=64,
+                                temp_coef=0.3, temp_every=1024, kv_from={i: i - 2 for i in range(2, nl, 4)},
+                                g_heads=s["heads"] // 2, g_dim=128, g_vdim=128, tau=16.0, rank=16,
+                                name=f"girulorn-{sz}", **moe)
+            yield "girulorn", lambda: GI.GirulornModel.load(gc, GI.synthetic_source(gc, 1), dev, torch.bfloat16)
+            pat = tuple("mamba2" if i % 4 == 3 else "parallel" for i in range(nl))
+            uc = VU.make_config(hidden=s["hidden"], vocab=V, pattern=pat, mlps=("moe",), heads=s["heads"],
+                                kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, chunk=args.arch_chunk,
+                                d_heads=s["heads"] // 2, d_kv_heads=max(1, s["heads"] // 4), d_dim=128, d_vdim=128,
+                                d_conv=4, m_heads=2 * s["hidden"] // 64, m_vdim=64, m_state=128, m_groups=1,
+                                m_norm_groups=1, m_conv=4, name=f"vugotar-{sz}", **moe)
+            yield "vugotar-moe", lambda: VU.VugotarModel.load(uc, VU.synthetic_source(uc, 1), dev, torch.bfloat16)
+        elif args.arch_bench == "vugotar":
             # attention + delta-rule layers with a state-space layer every fourth, dense feed-forwards; attention
             # heads as the Llama graph's (GQA 4:1, head size 128), delta rule with half as many heads of 128 x 128
             # states, state-space layer twice as wide as the model with 128 states per head

@@ -2,7 +2,7 @@
 // border, a window's edge or position 0, and an optional sink term in the denominator (ops/hybrid.py
 // masked_attention). Pools are token-major: keys [blocks, bs, G * dk], values [blocks, bs, G * dv], fp32 or bf16.
 // Every kernel also takes an AttnExtra: a learned sink score per head instead of 0, an additive bias looked up by the
-// distance between query and key (table [distances, H], the last row serving every larger distance), and a gate per
+// distance between query and key (table [H, distances], the last entry serving every larger distance), and a gate per
 // row and head whose sigmoid multiplies the head's output.
 //
 // attn_rows_kernel: one wave per (query row, query head). Keys are taken 64 at a time, one per lane: the lane forms
@@ -27,14 +27,14 @@ constexpr int DVU_MAX = 8;  // value columns per lane: heads of up to 512 number
 
 struct AttnExtra {
     const float* sink_v;  // [H] sink scores (null: 0 where a sink is asked for)
-    const float* bias;    // [nb, H] bias by distance (null: none)
+    const float* bias;    // [H, nb] bias by distance (null: none)
     int nb;
     const float* gate;    // pre-sigmoid gate of row r and head h at gate[r * ldg + h] (null: none)
     int ldg;
 };
 MX_DEV float sink_score(const AttnExtra& ex, int h) { return ex.sink_v ? ex.sink_v[h] : 0.f; }
 MX_DEV float dist_bias(const AttnExtra& ex, int dist, int H, int h) {
-    return ex.bias[(long)min(max(dist, 0), ex.nb - 1) * H + h];
+    return ex.bias[(long)h * ex.nb + min(max(dist, 0), ex.nb - 1)];
 }
 MX_DEV float gate_factor(const AttnExtra& ex, long row, int h) {
     return ex.gate ? 1.f / (1.f + expf(-ex.gate[row * ex.ldg + h])) : 1.f;
@@ -707,7 +707,7 @@ __global__ __launch_bounds__(256) void masked_softmax_kernel(const float* sc, vo
     const float* s = sc + row * nk;
     const float s0 = sink_v ? sink_v[h] : 0.f;
     const int d0 = pos - key0;  // distance of local key j: d0 - j
-    auto score = [&](int j) { return s[j] * scale + (bias ? bias[(long)min(d0 - j, nb - 1) * H + h] : 0.f); };
+    auto score = [&](int j) { return s[j] * scale + (bias ? bias[(long)h * nb + min(d0 - j, nb - 1)] : 0.f); };
     float m = sink ? s0 : -INFINITY;
     for (int j = a + threadIdx.x; j <= b; j += 256) m = fmaxf(m, score(j));
     m = block_max<256>(m, red);

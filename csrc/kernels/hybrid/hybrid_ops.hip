@@ -41,15 +41,17 @@ MX_DEV float block_sum_dyn(float v, float* red) {
 
 template <bool B16>
 __global__ __launch_bounds__(NT) void embed_rows_kernel(const void* table, int V, const int* tokens, float* out,
-                                                        int ldo, int accumulate, int C) {
+                                                        int ldo, int accumulate, int C, bf16_t* o16, int ld16) {
     const int t = blockIdx.x;
     int tok = tokens[t];
     if (tok < 0 || tok >= V) tok = 0;
     const long base = (long)tok * C;
     float* o = out + (long)t * ldo;
     for (int c = threadIdx.x; c < C; c += NT) {
-        const float v = ld_elem<B16>(table, base + c);
-        o[c] = accumulate ? o[c] + v : v;
+        float v = ld_elem<B16>(table, base + c);
+        if (accumulate) v += o[c];
+        o[c] = v;
+        if (o16) o16[(long)t * ld16 + c] = f32_to_bf16(v);
     }
 }
 
@@ -307,12 +309,23 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
     coef[i] = b ? sigmoid_acc(b[(long)t * ldb + h]) : s;
 }
 
-// out = exp(log_sigmoid(z + bias) * inv_tau) = sigmoid(z + bias)^(1 / tau)
+// out = exp(log_sigmoid(x) * inv_tau) = sigmoid(x)^(1 / tau) with x = z + bias, or, with a projection proj [R, C],
+// x = sum_r z[t, r] proj[r, c] + bias[c] (the second half of a low-rank projection, summed in fp32 in a fixed order)
 __global__ __launch_bounds__(NT) void channel_decay_kernel(const float* z, int ldz, const float* bias, float inv_tau,
-                                                           float* out, int C) {
+                                                           float* out, int C, const float* proj, int R) {
+    extern __shared__ float zr[];  // the token's R inputs of the projection
     const int c = blockIdx.y * NT + threadIdx.x, t = blockIdx.x;
+    if (proj) {
+        for (int r = threadIdx.x; r < R; r += NT) zr[r] = z[(long)t * ldz + r];
+        __syncthreads();
+    }
     if (c >= C) return;
-    const float x = z[(long)t * ldz + c] + (bias ? bias[c] : 0.f);
+    float x = bias ? bias[c] : 0.f;
+    if (proj) {
+        for (int r = 0; r < R; ++r) x += zr[r] * proj[(long)r * C + c];
+    } else {
+        x += z[(long)t * ldz + c];
+    }
     out[(long)t * C + c] = expf(-softplus_acc(-x) * inv_tau);
 }
 
@@ -465,11 +478,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int 
     if (!(cond)) return (int)hipErrorInvalidValue
 
 extern "C" int mxh_embed_rows(const void* table, int is16, int V, const int* tokens, float* out, int ldo,
-                              int accumulate, int T, int C, hipStream_t st) {
+                              int accumulate, bf16_t* o16, int ld16, int T, int C, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(table && tokens && out && C > 0 && V > 0 && ldo >= C);
-    if (is16) embed_rows_kernel<true><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C);
-    else embed_rows_kernel<false><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C);
+    MXH_CHECK(table && tokens && out && C > 0 && V > 0 && ldo >= C && (!o16 || ld16 >= C));
+    if (is16) embed_rows_kernel<true><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C, o16, ld16);
+    else embed_rows_kernel<false><<<T, NT, 0, st>>>(table, V, tokens, out, ldo, accumulate, C, o16, ld16);
     return (int)hipGetLastError();
 }
 
@@ -546,10 +559,12 @@ extern "C" int mxh_scan_coefs(const float* a, int lda, const float* b, int ldb, 
 }
 
 extern "C" int mxh_channel_decay(const float* z, int ldz, const float* bias, float inv_tau, float* out, int T, int C,
-                                 hipStream_t st) {
+                                 const float* proj, int R, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(z && out && C > 0 && ldz >= C && inv_tau > 0.f && C <= 65535 * NT);
-    channel_decay_kernel<<<dim3(T, (C + NT - 1) / NT), NT, 0, st>>>(z, ldz, bias, inv_tau, out, C);
+    MXH_CHECK(z && out && C > 0 && inv_tau > 0.f && C <= 65535 * NT);
+    MXH_CHECK(proj ? (R > 0 && R <= 8192 && ldz >= R) : ldz >= C);
+    channel_decay_kernel<<<dim3(T, (C + NT - 1) / NT), NT, proj ? R * sizeof(float) : 0, st>>>(z, ldz, bias, inv_tau, out,
+                                                                                            C, proj, R);
     return (int)hipGetLastError();
 }
 

@@ -142,8 +142,8 @@ LATENT_SIGS = {
 
 # libmxh.so (csrc/kernels/hybrid/): kernels of the hybrid attention / recurrent decoders (ops/hybrid.py)
 HYBRID_SIGS = {
-    # table, is16, V, tokens, out, ldo, accumulate, T, C, stream
-    "mxh_embed_rows": [P, I, I, P, P, I, I, I, I, P],
+    # table, is16, V, tokens, out, ldo, accumulate, out16, ld16, T, C, stream
+    "mxh_embed_rows": [P, I, I, P, P, I, I, P, I, I, I, P],
     # x, ldx, rows, w, offset, eps, out32, ld32, out16, ld16, M, C, stream
     "mxh_offset_norm": [P, I, P, P, F, F, P, I, P, I, I, I, P],
     # y, ldy, w, offset, eps, x, ldx, out16, ld16, T, C, stream
@@ -176,8 +176,8 @@ HYBRID_SIGS = {
     "mxh_unit_norm": [P, I, I, I, F, F, I, F, I, P],
     # a, lda, b, ldb, A_log, dt_bias, decay, coef, T, H, stream
     "mxh_scan_coefs": [P, I, P, I, P, P, P, P, I, I, P],
-    # z, ldz, bias, 1 / tau, out, T, C, stream
-    "mxh_channel_decay": [P, I, P, F, P, I, I, P],
+    # z, ldz, bias, 1 / tau, out, T, C, proj, R, stream
+    "mxh_channel_decay": [P, I, P, F, P, I, I, P, I, P],
     # k, ldk, q, ldq, v, ldv, decay, coef, skip, state, seq_state, positions, n_dec, pf_cu, n_pf, out, ldo, H, G, N, P,
     # delta, channel, q_scale, stream
     "mxh_state_scan": [P, I, P, I, P, I, P, P, P, P, P, P, I, P, I, P, I, I, I, I, I, I, I, F, P],

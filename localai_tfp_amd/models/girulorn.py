@@ -22,7 +22,8 @@ How a layer maps onto launches (T rows of a ragged engine step; hin is x in fp32
 
     y = hin W_in^T              every projection of the mixer that reads x, stacked into ONE GEMM (fp32 out)
     attention: head norms + temperature + paged append; masked attention (bias, sink, gate fused) -> cat
-    gla:       z = a1 W_a2^T (fp32); channel decay; state scan; head norm * silu(g) -> cat
+    gla:       channel decays (second decay projection in fp32 + bias + sigmoid^(1/tau)); state scan; head norm * silu(g)
+               -> cat
     o = cat W_o^T (fp32);  x += norm(o), hin <- x                                 ops/hybrid.py norm_add
     y = hin W_ff^T              router | shared gate, up | every expert's gate, up as ONE GEMM
     routing weights [T, E]; glu (shared); glu (experts, each scaled by its routing weight, 0 when not chosen) -> cat
@@ -233,9 +234,9 @@ class GirulornWeights:
     k_o: int
     q_norm: torch.Tensor | None = None
     k_norm: torch.Tensor | None = None
-    bias: torch.Tensor | None = None  # distance-bias table, one row per distance [ceil(bias_max) + 1, H]
+    bias: torch.Tensor | None = None  # distance-bias table, one entry per head and distance [H, ceil(bias_max) + 1]
     sink: torch.Tensor | None = None
-    a2: Dense | None = None  # fp32 in both modes
+    a2: torch.Tensor | None = None  # [rank, heads * dim], fp32 in both modes
     a2_b: torch.Tensor | None = None
     mix_norm: torch.Tensor | None = None
     norm2: torch.Tensor | None = None
@@ -275,7 +276,6 @@ class GirulornWorkspace:
         self.y = torch.empty((T * n_y,), **f32)
         self.o = torch.empty((T, C), **f32)
         self.q = torch.empty((T * n_q,), **m16)
-        self.z = torch.empty((T * n_dec,), **f32)
         self.decay = torch.empty((T * n_dec,), **f32)
         self.scan = torch.empty((T * n_scan,), **f32)
         self.cat = torch.zeros((T * k_cat,), **m16)  # zero: padded columns are read, never written
@@ -335,9 +335,11 @@ class GirulornModel:
     def weight_bytes(self) -> int:
         n = self.embed.numel() * self.embed.element_size() + self.head.w.numel() * self.head.w.element_size()
         for W in self.weights.values():
-            for dn in (W.w_in, W.w_o, W.a2, W.w_ff, W.w_down):
+            for dn in (W.w_in, W.w_o, W.w_ff, W.w_down):
                 if dn is not None:
                     n += dn.w.numel() * dn.w.element_size()
+            if W.a2 is not None:
+                n += W.a2.numel() * 4
         return n
 
     # ------------------------------------------------------------------ loading
@@ -394,7 +396,7 @@ class GirulornModel:
                 parts = [("q", t(p + "q", (H * dk, C))), ("k", t(p + "k", (H * dk, C))), ("v", t(p + "v", (H * dv, C))),
                          ("g", t(p + "g", (H * dv, C))), ("a1", t(p + "a1", (r, C)))]
                 w_o = along_k([t(p + "o", (C, H * dv))])
-                kw.update(a2=Dense(t(p + "a2", (H * dk, r)), None, dev, torch.float32), a2_b=f32(p + "a2.b", (H * dk,)),
+                kw.update(a2=t(p + "a2", (H * dk, r)).t().contiguous().to(dev), a2_b=f32(p + "a2.b", (H * dk,)),
                           mix_norm=f32(p + "norm", (dv,)))
             w_in, cols, n_in = stack(parts)
             f, q = L.mlp, f"l{i}.mlp."
@@ -429,14 +431,14 @@ class GirulornModel:
         b16 = self.dtype != torch.float32
         rag = HY.Ragged(fb)
         x = ws.x[:T]
-        HY.embed_rows(self.embed, fb.tokens, x)
+        hin = ws.hin[:T] if b16 else x  # what the GEMMs read: the residual itself, rounded in bf16 mode
+        x16 = hin if b16 else None
+        HY.embed_rows(self.embed, fb.tokens, x, out16=x16)
         if fb.embed_rows:
             for r0, e in fb.embed_rows:
                 x[r0:r0 + e.shape[0]].copy_(e)
-        hin = ws.hin[:T] if b16 else x  # what the GEMMs read: the residual itself, rounded in bf16 mode
-        x16 = hin if b16 else None
-        if b16:
-            hin.copy_(x)
+            if b16:
+                hin.copy_(x)
         o = ws.o[:T]
         for li, L in enumerate(cfg.layers):
             if fb.stop_layer is not None and li >= fb.stop_layer:
@@ -502,10 +504,8 @@ class GirulornModel:
         H, dk, dv = g.heads, g.dim, g.vdim
         c = W.cols
         nk, nv = H * dk, H * dv
-        z = ws.z[:T * nk].view(T, nk)
-        torch.mm(y[:, c["a1"]:c["a1"] + g.rank], W.a2.wt, out=z)  # fp32 x fp32: the decay's logits never see 16 bits
-        decay = ws.decay[:T * nk].view(T, nk)
-        HY.channel_decay(z, W.a2_b, g.tau, decay)
+        decay = ws.decay[:T * nk].view(T, nk)  # second projection (fp32: its logits never see 16 bits), bias, decay
+        HY.channel_decay(y[:, c["a1"]:c["a1"] + g.rank], W.a2_b, g.tau, decay, proj=W.a2)
         o = ws.scan[:T * nv].view(T, nv)
         HY.state_scan(y[:, c["k"]:c["k"] + nk], y[:, c["q"]:c["q"] + nk], y[:, c["v"]:c["v"] + nv], decay, None, None,
                       state, rag, o, H, H, dk, dv, delta=False, channel=True, q_scale=dk ** -0.5)

@@ -44,17 +44,22 @@ def _f32c(t: torch.Tensor, what: str):
 
 
 # ------------------------------------------------------------------------------------------------ embedding, norm
-def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, accumulate: bool = False):
-    """out[t] (=|+=) table[tokens[t]]; table fp32 or bf16 [V, C], out fp32 [T, C]."""
+def embed_rows(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+               out16: torch.Tensor | None = None):
+    """out[t] (=|+=) table[tokens[t]]; table fp32 or bf16 [V, C], out fp32 [T, C]; `out16` (bf16 [T, C]) also receives
+    the result, rounded (the operand of a GEMM that reads the residual itself)."""
     T, C = out.shape
     if T == 0:
         return out
     if not out.is_cuda:
         rows = table[tokens.long()].float()
         out.add_(rows) if accumulate else out.copy_(rows)
+        if out16 is not None:
+            out16.copy_(out)
         return out
     N.kcall("mxh_embed_rows", table.data_ptr(), _is16(table), table.shape[0], tokens.data_ptr(), out.data_ptr(),
-            out.stride(0), int(accumulate), T, C, N.stream_ptr())
+            out.stride(0), int(accumulate), N.ptr(out16), out16.stride(0) if out16 is not None else 0, T, C,
+            N.stream_ptr())
     return out
 
 
@@ -102,10 +107,11 @@ def norm_add(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor, out1
 
 # ------------------------------------------------------------------------------------------------ attention
 def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
-    """Expands a bucketed distance-bias table rel [B, H] into one row per distance: out [ceil(far) + 1, H] fp32 with
-    out[n] = rel[bucket(n)], bucket(n) = n for n < B/2, else min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(far / (B/2))
-    * (B - B/2))). Every distance >= far lands in the last bucket, so the last row serves all of them
-    (`masked_attention` clamps the distance to the table)."""
+    """Expands a bucketed distance-bias table rel [B, H] into one entry per distance and head: out [H, ceil(far) + 1]
+    fp32 (a head's entries contiguous: neighbouring keys are neighbouring numbers) with out[h, n] = rel[bucket(n), h],
+    bucket(n) = n for n < B/2, else min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(far / (B/2)) * (B - B/2))). Every
+    distance >= far lands in the last bucket, so the last entry serves all of them (`masked_attention` clamps the
+    distance to the table)."""
     B = rel.shape[0]
     half = B // 2
     if half < 1 or far <= half:
@@ -119,7 +125,7 @@ def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
         if abs(v - round(v)) < 1e-9:  # a whole number up to the rounding of the logarithms
             v = round(v)
         idx.append(min(B - 1, half + int(math.floor(v))))
-    return rel.float()[torch.tensor(idx, device=rel.device)].contiguous()
+    return rel.float()[torch.tensor(idx, device=rel.device)].t().contiguous()
 
 
 def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, positions: torch.Tensor, H: int,
@@ -201,7 +207,7 @@ def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, s
     lo = (i // chunk) * chunk if chunk else (i - window + 1).clamp(min=0) if window else torch.zeros_like(i)
     vis = (j <= i) & (j >= lo)
     if bias is not None:
-        s = s + bias.float()[(i - j).clamp(0, bias.shape[0] - 1)].permute(2, 0, 1)
+        s = s + bias.float()[:, (i - j).clamp(0, bias.shape[1] - 1)]
     s = s.masked_fill(~vis[None], float("-inf"))
     m = s.max(-1, keepdim=True).values
     if sink:
@@ -269,7 +275,7 @@ def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window
         sc = bmm_f32(qh.view(G, rep * n2, dk), kh.transpose(1, 2))
         pw = torch.empty((G, rep * n2, nk), dtype=md, device=dev)
         N.kcall("mxh_masked_softmax", sc.data_ptr(), pw.data_ptr(), i16, H * n2, n2, nk, a, key0, float(scale),
-                int(chunk), int(window), int(sink), N.ptr(sink_v), N.ptr(bias), bias.shape[0] if bias is not None else 0,
+                int(chunk), int(window), int(sink), N.ptr(sink_v), N.ptr(bias), bias.shape[1] if bias is not None else 0,
                 H, st)
         o = bmm_f32(pw, vh)
         orow = out[a - p0:]
@@ -285,7 +291,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key /
     value head h // (H / G). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
     max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
-    [H] adds exp(sink[h]). `bias` (fp32 [L, H], contiguous) adds bias[min(i - j, L - 1), h] to the scaled score.
+    [H] adds exp(sink[h]). `bias` (fp32 [H, L], contiguous) adds bias[h, min(i - j, L - 1)] to the scaled score.
     `gate` (fp32 [T, H], may be a column slice) multiplies head h's output of row t by sigmoid(gate[t, h]). out
     [T, H*dv] (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32
     or bf16 operands; scores, softmax and the accumulators are fp32.
@@ -304,9 +310,9 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     sink = sink_v is not None or bool(sink)
     if sink_v is not None and (sink_v.dtype != torch.float32 or sink_v.numel() != H or not sink_v.is_contiguous()):
         raise TypeError("masked_attention: one fp32 sink per query head")
-    if bias is not None and (bias.dtype != torch.float32 or bias.dim() != 2 or bias.shape[1] != H
+    if bias is not None and (bias.dtype != torch.float32 or bias.dim() != 2 or bias.shape[0] != H
                              or not bias.is_contiguous()):
-        raise TypeError("masked_attention: the distance bias is a contiguous fp32 [distances, H] table")
+        raise TypeError("masked_attention: the distance bias is a contiguous fp32 [H, distances] table")
     if gate is not None and (gate.dtype != torch.float32 or gate.shape != (T, H) or gate.stride(1) != 1):
         raise TypeError("masked_attention: the gate is fp32 [T, H]")
     nd = rag.n_dec
@@ -331,7 +337,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     bs = kc.shape[1]
     st = N.stream_ptr()
     common = (H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale))
-    nb = bias.shape[0] if bias is not None else 0
+    nb = bias.shape[1] if bias is not None else 0
     ldg = gate.stride(0) if gate is not None else 0
     extra = (N.ptr(sink_v), N.ptr(bias), nb)  # the gate pointer moves with the rows a launch serves
     mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
@@ -473,21 +479,30 @@ def scan_coefs(a: torch.Tensor, b: torch.Tensor | None, A_log: torch.Tensor, dt_
             A_log.data_ptr(), dt_bias.data_ptr(), decay.data_ptr(), coef.data_ptr(), T, H, N.stream_ptr())
 
 
-def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: torch.Tensor):
-    """out = sigmoid(z + bias)^(1 / tau), computed as exp(log_sigmoid(z + bias) / tau): the per-channel decay of gated
-    linear attention. z fp32 [T, C] (column slice allowed), bias fp32 [C], out fp32 [T, C] contiguous."""
-    T, C = z.shape
+def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: torch.Tensor,
+                  proj: torch.Tensor | None = None):
+    """out = sigmoid(x)^(1 / tau), computed as exp(log_sigmoid(x) / tau): the per-channel decay of gated linear
+    attention. x = z + bias with z fp32 [T, C]; or, with `proj` (fp32 [R, C], contiguous), x = z proj + bias with z
+    fp32 [T, R]: the second half of a low-rank projection, done in fp32 inside the same kernel. z may be a column
+    slice; bias fp32 [C]; out fp32 [T, C] contiguous."""
+    T, C = out.shape
     if T == 0:
         return out
+    if z.shape != ((T, proj.shape[0]) if proj is not None else (T, C)) or (proj is not None and proj.shape[1] != C):
+        raise ValueError("channel_decay: z is [T, C], or [T, R] beside a projection [R, C]")
     if not z.is_cuda:
-        x = z.float() + bias.float() if bias is not None else z.float()
+        x = z.float() @ proj.float() if proj is not None else z.float()
+        if bias is not None:
+            x = x + bias.float()
         out.copy_(torch.exp(F.logsigmoid(x) / tau))
         return out
     _f32c(z, "channel_decay")
     if not out.is_contiguous() or out.dtype != torch.float32 or tau <= 0:
         raise ValueError("channel_decay: contiguous fp32 output, tau > 0")
+    if proj is not None and (proj.dtype != torch.float32 or not proj.is_contiguous()):
+        raise TypeError("channel_decay: the projection is a contiguous fp32 [R, C] matrix")
     N.kcall("mxh_channel_decay", z.data_ptr(), z.stride(0), N.ptr(bias), float(1.0 / tau), out.data_ptr(), T, C,
-            N.stream_ptr())
+            N.ptr(proj), proj.shape[0] if proj is not None else 0, N.stream_ptr())
     return out
 
 

@@ -84,9 +84,9 @@ def test_distance_buckets():
     for rows, far in ((12, 40.0), (2, 3.0), (30, 1000.0), (32, 128.0), (64, 512.0), (8, 4.5), (16, 64.0)):
         rel = torch.arange(rows * 3, dtype=torch.float32).reshape(rows, 3)
         lut = HY.log_bucket_table(rel, far)
-        assert lut.shape[0] >= far and lut.shape[1] == 3
-        for n in range(lut.shape[0] + 20):
-            assert lut[min(n, lut.shape[0] - 1), 1] == rel[O.distance_bucket(n, rows, far), 1], (rows, far, n)
+        assert lut.shape[1] >= far and lut.shape[0] == 3
+        for n in range(lut.shape[1] + 20):
+            assert lut[1, min(n, lut.shape[1] - 1)] == rel[O.distance_bucket(n, rows, far), 1], (rows, far, n)
     assert O.distance_bucket(64, 64, 512.0) == 40 and O.distance_bucket(63, 64, 512.0) == 39
     assert O.distance_bucket(127, 32, 128.0) == 31 and O.distance_bucket(10 ** 6, 32, 128.0) == 31
 
@@ -217,6 +217,11 @@ def test_channel_decay_scan_in_portions(dev, H, N, P):
     dec = torch.empty(n, H * N, device=dev)
     HY.channel_decay(z.to(dev), zb.to(dev), tau, dec)
     close(dec, alpha, 1e-5)
+    for R in (3, 16, 300):  # the same with the second half of a low-rank projection inside
+        lo, pr = torch.randn(n, R + 1, generator=g), torch.randn(R, H * N, generator=g) * R ** -0.5
+        dec2 = torch.empty(n, H * N, device=dev)
+        HY.channel_decay(lo.to(dev)[:, 1:], zb.to(dev), tau, dec2, proj=pr.to(dev))
+        close(dec2, torch.sigmoid(lo[:, 1:].double() @ pr.double() + zb.double()).pow(1.0 / tau), 1e-5)
     state = torch.full((2, H, P, N), 4.0, device=dev)  # slot 1 is dirty: position 0 must not read it
     out = torch.empty(n, H * P, device=dev)
     for n_dec, chunks, at in steps_of(n, [9, 1, 2, 1, 1, 20, 3, 2, 1, 5]):
