@@ -15,8 +15,6 @@
 // S[n][p] <- a_t[n] S[n][p] + k_t[n] u[p]. A missing write strength means 1; q_t is multiplied by q_scale when staged.
 #include "../mx_common.h"
 
-#include <type_traits>
-
 namespace {
 
 template <int CTRL>
@@ -100,19 +98,20 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
     // TB tokens' k, q, value, decay and write strength wait in registers while the TB tokens before them are worked
     // on, then move to LDS: memory latency is paid once per TB steps, and a barrier too
     float st_kq[KQ_PT], st_v[V_PT], st_ac = 0.f;
-    // FULL: a round of TB tokens, every load unconditional (all in flight together); otherwise only the round's tokens
-    // are asked for (a decode row wants one token's numbers, not TB copies of them)
-    auto fetch_some = [&](int c, auto full) {
-        constexpr bool FULL = decltype(full)::value;
+    // a round's loads are unconditional (clamped addresses, all in flight together) except that whole groups of NT
+    // loads beyond the round's tokens are skipped by a block-uniform test: a decode row asks for one token's numbers,
+    // not TB copies of them
+    auto fetch = [&](int c) {
         const int r0 = row0 + c * TB;
-        const int ntc = FULL ? TB : min(TB, n - c * TB);
+        const int ntc = min(TB, n - c * TB);
 #pragma unroll
         for (int i = 0; i < KQ_PT; ++i) {
-            const int idx = threadIdx.x + i * NT;
-            const int tt = idx / (NW * NP), w = (idx / NP) % NW, e = idx % NP;
             float x = 0.f;
-            if (FULL || tt < ntc) {
-                const long row = r0 + tt;
+            const int idx = threadIdx.x + i * NT;
+            const int e = idx % NP;
+            if (i * NT < ntc * NW * NP) {
+                const int tt = idx / (NW * NP), w = (idx / NP) % NW;
+                const long row = min(r0 + tt, last);
                 const int ec = min(e, N - 1);
                 if (CHD && w == 2) x = decay[row * ((long)H * N) + (long)h * N + ec];
                 else x = w ? qp[row * ldq + ec] * q_scale : kp[row * ldk + ec];
@@ -121,20 +120,19 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
         }
 #pragma unroll
         for (int i = 0; i < V_PT; ++i) {
-            const int idx = min(threadIdx.x + i * NT, TB * COLS - 1);
-            const int tt = idx / COLS, cc = idx % COLS;
-            st_v[i] = (FULL || tt < ntc)
-                          ? v[(long)(r0 + tt) * ldv + (long)h * P + min((int)blockIdx.x * COLS + cc, P - 1)] : 0.f;
+            st_v[i] = 0.f;
+            if (i * NT < ntc * COLS) {
+                const int idx = min(threadIdx.x + i * NT, TB * COLS - 1);
+                const int tt = idx / COLS, cc = idx % COLS;
+                const long row = min(r0 + tt, last);
+                st_v[i] = v[row * ldv + (long)h * P + min((int)blockIdx.x * COLS + cc, P - 1)];
+            }
         }
-        if (threadIdx.x < 2 * ntc) {
+        if (threadIdx.x < 2 * TB) {
             const long row = min(r0 + (int)threadIdx.x / 2, last);
             if (threadIdx.x & 1) st_ac = coef ? coef[row * H + h] : 1.f;
             else st_ac = CHD ? 1.f : decay[row * H + h];
         }
-    };
-    auto fetch = [&](int c) {
-        if (n - c * TB >= TB) fetch_some(c, std::true_type{});
-        else fetch_some(c, std::false_type{});
     };
     auto publish = [&](int b) {
 #pragma unroll

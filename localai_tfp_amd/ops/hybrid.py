@@ -116,16 +116,11 @@ def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
     half = B // 2
     if half < 1 or far <= half:
         raise ValueError("log_bucket_table: at least two rows, and the far distance lies beyond the exact half")
-    idx = []
-    for n in range(int(math.ceil(far)) + 1):
-        if n < half:
-            idx.append(n)
-            continue
-        v = math.log(n / half) / math.log(far / half) * (B - half)
-        if abs(v - round(v)) < 1e-9:  # a whole number up to the rounding of the logarithms
-            v = round(v)
-        idx.append(min(B - 1, half + int(math.floor(v))))
-    return rel.float()[torch.tensor(idx, device=rel.device)].t().contiguous()
+    n = torch.arange(int(math.ceil(far)) + 1, dtype=torch.float64)
+    v = torch.log(n.clamp(min=half) / half) / math.log(far / half) * (B - half)
+    v = torch.where((v - v.round()).abs() < 1e-9, v.round(), v)  # a whole number up to the rounding of the logarithms
+    idx = torch.where(n < half, n, (half + v.floor()).clamp(max=B - 1)).long()
+    return rel.float()[idx.to(rel.device)].t().contiguous()
 
 
 def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, positions: torch.Tensor, H: int,
