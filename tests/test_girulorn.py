@@ -357,6 +357,24 @@ def test_peaked_attention_far_keys_and_long_decode(dev, dt, tol):
     close(got, want, tol * 2, rms=dt == "bfloat16")
 
 
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
+@pytest.mark.parametrize("dim,vdim,heads,kv", [(64, 128, 8, 2), (128, 64, 3, 1), (64, 64, 20, 1)])
+def test_matrix_core_head_sizes_through_the_engine(dev, dt, tol, dim, vdim, heads, kv):
+    """Head sizes of 64 / 128 (bf16 prompts and decoded rows run on the matrix cores, up to 16 query heads per key
+    head; 20 take the row kernel): a prompt longer than the bias table, portions that end inside 16-row tiles, decoded
+    rows behind enough keys to be split into partitions, a borrowing layer."""
+    kw = dict(hidden=128, vocab=211, pattern=("attention", "gla", "attention"), kv_from={2: 0}, heads=heads, kv_heads=kv,
+              dim=dim, vdim=vdim, scale=1.5 * dim ** -0.5, bias_max=200.0, bias_rows=16, temp_coef=0.3, temp_every=100,
+              g_heads=2, g_dim=64, g_vdim=64, tau=8.0, rank=4, experts=4, top=2, expert_ff=64, shared_ff=64)
+    cfg, tensors, model = build(dev, dt, seed=17, **kw)
+    t = toks(330, cfg.vocab, 9)
+    want = oracle(cfg, tensors, t)
+    eng = engine(model, max_tokens=336, seqs=2)
+    b16 = dt == "bfloat16"
+    close(run_cuts(eng, "x", t, [203, 17, 2, 41, 1, 1, 1, 33] + [1] * 31), want, tol, b16)
+    close(run_cuts(eng, "y", t[:100], [100]), want[:100], tol, b16)
+
+
 # ------------------------------------------------------------------------------------------------ serving path
 @pytest.mark.parametrize("dev,dt", [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu)])
 @pytest.mark.parametrize("native", [False, True])
