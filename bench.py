@@ -248,8 +248,8 @@ def run_arch_bench(args) -> int:
             moe = dict(experts=8, top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 2)
             gc = GI.make_config(hidden=s["hidden"], vocab=V, pattern=pat, heads=s["heads"],
                                 kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, bias_max=4096.0, bias_rows=64,
-                                temp_coef=0.3, temp_every=1024, kv_from={i: i - 2 for i in range(2, nl, 4)},
-                                g_heads=s["heads"] // 2, g_dim=128, g_vdim=128, tau=16.0, rank=16,
+                                temp_coef=0.25, temp_every=1024, kv_from={i: i - 2 for i in range(2, nl, 4)},
+                                g_heads=s["heads"] // 2, g_dim=128, g_vdim=128, tau=12.0, rank=32,
                                 name=f"girulorn-{sz}", **moe)
             yield "girulorn", lambda: GI.GirulornModel.load(gc, GI.synthetic_source(gc, 1), dev, torch.bfloat16)
             pat = tuple("mamba2" if i % 4 == 3 else "parallel" for i in range(nl))

@@ -214,11 +214,11 @@ SYNTHETIC = {
     "girulorn-tiny": dict(hidden=256, vocab=512, pattern=("attention", "gla", "attention"), kv_from={2: 0}),
     "girulorn-1b": dict(hidden=2048, vocab=32000, pattern=("attention", "gla") * 8, heads=16, kv_heads=4, dim=128,
                         vdim=128, bias_max=4096.0, bias_rows=64, temp_every=1024, g_heads=16, g_dim=128, g_vdim=128,
-                        tau=16.0, rank=16, experts=8, top=2, expert_ff=2048, shared_ff=4096,
+                        tau=12.0, rank=32, experts=8, top=2, expert_ff=2048, shared_ff=4096,
                         kv_from={i: i - 2 for i in range(2, 16, 4)}),
     "girulorn-7b": dict(hidden=4096, vocab=32000, pattern=("attention", "gla") * 16, heads=32, kv_heads=8, dim=128,
                         vdim=128, bias_max=4096.0, bias_rows=64, temp_every=1024, g_heads=32, g_dim=128, g_vdim=128,
-                        tau=16.0, rank=16, experts=8, top=2, expert_ff=3584, shared_ff=7168,
+                        tau=12.0, rank=32, experts=8, top=2, expert_ff=3584, shared_ff=7168,
                         kv_from={i: i - 2 for i in range(2, 32, 4)}),
 }
 

@@ -348,7 +348,7 @@ def test_peaked_attention_far_keys_and_long_decode(dev, dt, tol):
     """A large score scale makes single keys dominate, so a lost or shifted key anywhere in a long prompt (page
     borders, position 0, beyond the bias table's last distance) moves the logits; then 70 tokens decoded one by one
     while the temperature steps and the decayed state is carried on."""
-    kw = dict(SHAPES["plain"], scale=2.5, bias_max=100.0, temp_every=64)
+    kw = dict(SHAPES["plain"], scale=2.5, bias_max=100.0, temp_every=50)
     cfg, tensors, model = build(dev, dt, seed=21, **kw)
     t = toks(260, cfg.vocab, 8)
     want = oracle(cfg, tensors, t)
