@@ -182,6 +182,27 @@ def test_attention_bias_buckets_pages_sinks_and_gates(dev, dt, tol, gemm_rows, m
     close(got, want, tol * b16)
 
 
+@pytest.mark.gpu
+def test_matrix_core_kernels_agree_with_the_row_kernels(monkeypatch):
+    """bf16 runs round their operands, so the oracle bounds them only loosely; the matrix-core kernels (prompt portions,
+    decoded rows, partitions) and the row kernels read the same rounded operands and must agree to a few bf16 steps: a
+    wrong bias entry, sink or gate for any head would show at once."""
+    plant = [(79, 40), (119, 80), (120, 119), (121, 120), (95, 81), (149, 12), (60, 60), (39, 0), (41, 39), (140, 100)]
+    far = [(270, 3), (280, 127), (281, 128), (299, 255), (290, 256), (295, 295)]
+    cases = [((H, G, dk, dv, 150, [37, 2, 41, 1, 17, 22, 1, 29], 16, 0.5, plant), {}) for H, G, dk, dv in
+             ((4, 2, 64, 64), (8, 2, 128, 128), (2, 2, 64, 128), (6, 3, 128, 64), (5, 1, 64, 64), (16, 1, 64, 64))]
+    cases += [((4, 1, 64, 64, 300, [200, 60] + [1] * 40, 16, 1.0, far), dict(rows=20, far=290.0)),
+              ((7, 1, 128, 128, 300, [100, 100, 59] + [1] * 41, 16, 0.5, far), dict(sink_shift=1.0, rows=6, far=9.0))]
+    for args, kw in cases:
+        out = []
+        for rows_min in (16, 0):  # 0: the matrix-core kernels are off
+            monkeypatch.setattr(HY, "MFMA_MIN_ROWS", rows_min)
+            got, want = _bias_attention_case("cuda", "bfloat16", *args, rel_scale=3.0, **kw)
+            out.append(got.double().cpu())
+        assert (out[0] - out[1]).abs().max().item() < 0.04, args[:4]  # values of up to 4: 1/64 is one bf16 step
+        close(out[0], want, 0.06)
+
+
 @pytest.mark.parametrize("dev", DEVS)
 def test_learned_sink_takes_or_leaves_the_weight(dev):
     """A large sink score holds the denominator (outputs shrink towards zero), a very negative one leaves the plain
