@@ -391,6 +391,32 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
                 sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, sacc[t], 0, 0, 0);
             }
         }
+        // ---- bias by distance: row 4g + i against key 16t + col lies d0 + i - 16t keys back. When every distance
+        // of the wave's 16 rows against the tile's 64 keys lies inside the table (a wave-uniform test) the 16 entries
+        // are read at constant offsets from one address; the diagonal tile and tiles beyond the table clamp ----
+        if (ex.bias) {
+            const float* bp = ex.bias + (size_t)hq * ex.nb;
+            const int d0 = p0 + row_q0 + 4 * g - kt0 - col;
+            const int dmin = p0 + row_q0 - (kt0 + KT - 1), dmax = p0 + row_q0 + 15 - kt0;
+            if (dmin >= 0 && dmax < ex.nb) {
+                const float* pp = bp + d0;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sacc[t][i] = sacc[t][i] * qs + pp[i - 16 * t] * LOG2E_;
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        sacc[t][i] = sacc[t][i] * qs + bp[min(max(d0 + i - 16 * t, 0), ex.nb - 1)] * LOG2E_;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sacc[t][i] *= qs;
+        }
         // ---- mask + online softmax in base 2 (rows 4g + i, keys 16t + col) ----
         float alpha[4];
 #pragma unroll
@@ -401,8 +427,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int kp = kt0 + 16 * t + col;
-                float v = sacc[t][i] * qs;
-                if (ex.bias) v += dist_bias(ex, qpos - kp, H, hq) * LOG2E_;
+                float v = sacc[t][i];
                 if (kp > qpos || kp < lo_row[i] || qi >= n) v = -INFINITY;
                 sacc[t][i] = v;
                 mx = fmaxf(mx, v);
@@ -552,6 +577,26 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
                                                                   0, 0, 0);
         }
         if (kt0 + KT < kv_end) load_tile(kt0 + KT);
+        // bias by distance: every row (query head) of the tile is at the same position, key 16t + col lies
+        // qpos - kt0 - col - 16t keys back; each head has its own table row
+        if (ex.bias) {
+            const int d0 = qpos - kt0 - col;
+            const bool inside = qpos - (kt0 + KT - 1) >= 0 && qpos - kt0 < ex.nb;  // wave-uniform: no clamps needed
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float* bp = ex.bias + (size_t)hrow[i] * ex.nb;
+#pragma unroll
+                for (int t = 0; t < KT / 16; ++t) {
+                    const int d = inside ? d0 - 16 * t : min(max(d0 - 16 * t, 0), ex.nb - 1);
+                    sacc[t][i] = sacc[t][i] * qs + bp[d] * LOG2E_;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int t = 0; t < KT / 16; ++t) sacc[t][i] *= qs;
+        }
         float alpha[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -559,8 +604,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
 #pragma unroll
             for (int t = 0; t < KT / 16; ++t) {
                 const int kp = kt0 + 16 * t + col;
-                float v = sacc[t][i] * qs;
-                if (ex.bias) v += dist_bias(ex, qpos - kp, H, hrow[i]) * LOG2E_;
+                float v = sacc[t][i];
                 if (kp >= kv_end) v = -INFINITY;
                 sacc[t][i] = v;
                 mx = fmaxf(mx, v);

@@ -140,8 +140,8 @@ class GirulornConfig:
                                     None if src is None else int(src))
                 _need(mixer.heads % mixer.kv_heads == 0, f"layer {i}: heads are a multiple of kv_heads")
                 _need(mixer.temp_every >= 1, f"layer {i}: q_temp.every >= 1")
-                _need(mixer.bias_rows >= 2 and mixer.bias_rows % 2 == 0 and mixer.bias_max > mixer.bias_rows // 2,
-                      f"layer {i}: an even number of bias rows, bias_max beyond the exact half")
+                _need(mixer.bias_rows >= 2 and mixer.bias_max > mixer.bias_rows // 2,
+                      f"layer {i}: at least two bias rows, bias_max beyond the exact half")
                 if mixer.kv_from is not None:
                     j = mixer.kv_from
                     _need(0 <= j < i and layers[j].type == "attention" and layers[j].mixer.kv_from is None,

@@ -308,6 +308,27 @@ def test_prompt_portions_and_decoding(dev, dt, tol, shape):
 
 
 @pytest.mark.parametrize("dev,dt,tol", RUNS)
+@pytest.mark.parametrize("kind", ["gla", "attention"])
+def test_models_of_one_kind_of_layer(dev, dt, tol, kind):
+    """Recurrent layers only (the paged pool is empty, blocks are bookkeeping) and attention layers only (the state
+    slots hold nothing), the second with a table of an odd number of rows and no feed-forward anywhere."""
+    kw = dict(SHAPES["plain"], pattern=(kind,) * 3, kv_from={2: 1} if kind == "attention" else None)
+    if kind == "attention":
+        kw.update(mlps=(None,), bias_rows=7, bias_max=11.0)
+    cfg, tensors, model = build(dev, dt, seed=13, **kw)
+    assert (model.cache_ranks() == []) == (kind == "gla")
+    t = toks(60, cfg.vocab, 3)
+    want = oracle(cfg, tensors, t)
+    ec = EngineConfig(max_num_seqs=2, max_batched_tokens=64, max_model_len=64, block_size=16, use_graphs=False,
+                      overlap=False, native_scheduler=False, logits_rows=64, gemm_autotune=False,
+                      num_blocks=0 if kind == "gla" else 9)
+    eng = LLMEngine(model, ByteTokenizer(cfg.vocab), ec)
+    b16 = dt == "bfloat16"
+    close(run_cuts(eng, "a", t, [60]), want, tol, b16)
+    close(run_cuts(eng, "b", t, [7, 2, 30] + [1] * 21), want, tol, b16)
+
+
+@pytest.mark.parametrize("dev,dt,tol", RUNS)
 def test_residual_after_every_layer(dev, dt, tol):
     cfg, tensors, model = build(dev, dt, seed=9, **SHAPES["plain"])
     t = toks(30, cfg.vocab, 2)
