@@ -102,29 +102,30 @@ __global__ __launch_bounds__(NT) void offset_norm_kernel(const float* x, int ldx
     }
 }
 
-// x[t] += y[t] / rms(y[t]) * (offset + w); o16 (optional) = the new x[t] rounded. One block per row, the row of y kept
-// in registers when it fits.
-__global__ __launch_bounds__(NT) void norm_add_kernel(const float* y, int ldy, const float* w, float offset, float eps,
-                                                      float* x, int ldx, bf16_t* o16, int ld16, int C) {
-    __shared__ float red[NT / 64];
-    const int i = blockIdx.x;
+// x[t] += y[t] / rms(y[t]) * (offset + w); o16 (optional) = the new x[t] rounded. One block per row (256 or 1024
+// threads: the launcher keeps the loads per thread few), the row of y kept in registers when it fits.
+template <int RK>
+__global__ __launch_bounds__(1024) void norm_add_kernel(const float* y, int ldy, const float* w, float offset, float eps,
+                                                        float* x, int ldx, bf16_t* o16, int ld16, int C) {
+    __shared__ float red[16];
+    const int i = blockIdx.x, nt = blockDim.x;
     const float* yr = y + (long)i * ldy;
     float* xr = x + (long)i * ldx;
-    const bool cached = C <= NT * RC;
-    float keep[RC], wk[RC], xk[RC];
+    const bool cached = C <= nt * RK;
+    float keep[RK], wk[RK], xk[RK];
     float ss = 0.f;
     if (cached) {
 #pragma unroll
-        for (int k = 0; k < RC; ++k) {  // clamped addresses: straight-line loads, all in flight together
-            const int c = min((int)threadIdx.x + k * NT, C - 1);
+        for (int k = 0; k < RK; ++k) {  // clamped addresses: straight-line loads, all in flight together
+            const int c = min((int)threadIdx.x + k * nt, C - 1);
             const float v = yr[c];
             wk[k] = w[c];
             xk[k] = xr[c];
-            keep[k] = (int)threadIdx.x + k * NT < C ? v : 0.f;
+            keep[k] = (int)threadIdx.x + k * nt < C ? v : 0.f;
             ss += keep[k] * keep[k];
         }
     } else {
-        for (int c = threadIdx.x; c < C; c += NT) {
+        for (int c = threadIdx.x; c < C; c += nt) {
             const float v = yr[c];
             ss += v * v;
         }
@@ -133,8 +134,8 @@ __global__ __launch_bounds__(NT) void norm_add_kernel(const float* y, int ldy, c
     const float sc = 1.f / sqrtf(ss / (float)C + eps);
     if (cached) {
 #pragma unroll
-        for (int k = 0; k < RC; ++k) {
-            const int c = threadIdx.x + k * NT;
+        for (int k = 0; k < RK; ++k) {
+            const int c = threadIdx.x + k * nt;
             if (c < C) {
                 const float v = xk[k] + keep[k] * sc * (offset + wk[k]);
                 xr[c] = v;
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(NT) void norm_add_kernel(const float* y, int ldy, c
         }
         return;
     }
-    for (int c = threadIdx.x; c < C; c += NT) {
+    for (int c = threadIdx.x; c < C; c += nt) {
         const float v = xr[c] + yr[c] * sc * (offset + w[c]);
         xr[c] = v;
         if (o16) o16[(long)i * ld16 + c] = f32_to_bf16(v);
@@ -498,7 +499,9 @@ extern "C" int mxh_norm_add(const float* y, int ldy, const float* w, float offse
                             bf16_t* o16, int ld16, int T, int C, hipStream_t st) {
     if (T <= 0) return 0;
     MXH_CHECK(y && w && x && C > 0 && ldy >= C && ldx >= C && (!o16 || ld16 >= C));
-    norm_add_kernel<<<T, NT, 0, st>>>(y, ldy, w, offset, eps, x, ldx, o16, ld16, C);
+    if (C <= 1024) norm_add_kernel<4><<<T, 256, 0, st>>>(y, ldy, w, offset, eps, x, ldx, o16, ld16, C);
+    else if (C <= 4096) norm_add_kernel<4><<<T, 1024, 0, st>>>(y, ldy, w, offset, eps, x, ldx, o16, ld16, C);
+    else norm_add_kernel<16><<<T, 1024, 0, st>>>(y, ldy, w, offset, eps, x, ldx, o16, ld16, C);
     return (int)hipGetLastError();
 }
 

@@ -68,7 +68,7 @@ def oracle(cfg, tensors, tokens, layers=None):
 def test_output_norm_and_residual_add(dev):
     g = torch.Generator().manual_seed(1)
     eps = 0.3  # a large eps shows whether it sits inside the root
-    for M, C in ((5, 72), (2, 4500)):  # the second is wider than a block keeps in registers
+    for M, C in ((5, 72), (3, 1100), (2, 4500), (2, 17000)):  # the last is wider than a block keeps in registers
         y, x = torch.randn(M, C + 2, generator=g) * 3, torch.randn(M, C, generator=g)
         w = 1.0 + 0.2 * torch.randn(C, generator=g)
         want = x.double() + O.rms_norm(y[:, 2:].double(), w, eps)
