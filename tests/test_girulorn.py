@@ -417,6 +417,70 @@ def test_matrix_core_head_sizes_through_the_engine(dev, dt, tol, dim, vdim, head
     close(run_cuts(eng, "y", t[:100], [100]), want[:100], tol, b16)
 
 
+def _random_shape(rng):
+    nl = rng.randint(2, 6)
+    pattern, kv_from, owners = [], {}, []
+    for i in range(nl):
+        kind = rng.choice(["attention", "gla"])
+        pattern.append(kind)
+        if kind == "attention":
+            if owners and rng.random() < 0.4:
+                kv_from[i] = rng.choice(owners)
+            else:
+                owners.append(i)
+    kv, rows, experts = rng.choice([1, 2, 3, 4]), rng.choice([2, 4, 8, 16, 32, 64]), rng.choice([2, 3, 4, 8, 16])
+    return dict(hidden=rng.choice([64, 96, 160]), vocab=rng.choice([97, 256, 1000]), pattern=tuple(pattern),
+                kv_from=kv_from, heads=kv * rng.choice([1, 2, 3, 6]), kv_heads=kv, dim=rng.choice([16, 32, 48, 64, 128]),
+                vdim=rng.choice([16, 32, 64, 128]), scale=rng.choice([0.05, 0.1, 0.2]),
+                bias_max=float(max(rows // 2 + 1, rng.choice([3, 30, 120, 500]))), bias_rows=rows,
+                temp_coef=rng.choice([0.0, 0.1, 0.5]), temp_every=rng.choice([1, 7, 64]), g_heads=rng.choice([1, 2, 4]),
+                g_dim=rng.choice([16, 32, 48, 64, 128]), g_vdim=rng.choice([16, 32, 96]), tau=rng.choice([1.0, 4.0, 64.0]),
+                rank=rng.choice([1, 4, 16]), mlps=tuple(rng.choice(["moe", "moe", None]) for _ in range(rng.randint(1, 3))),
+                experts=experts, top=rng.randint(1, experts), expert_ff=rng.choice([16, 40]),
+                shared_ff=rng.choice([0, 32, 96]), eps=rng.choice([1e-6, 1e-5]))
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_configurations_and_schedules(dev, seed):
+    """Drawn sizes, layer orders and borrowings; five requests fed through four live slots in drawn portions (single
+    tokens beside portions of up to 150, requests left out of steps, blocks and slots handed on) in a pool that holds
+    the four largest but not all five. fp32 only: every position agrees with the oracle."""
+    import random
+    rng = random.Random(seed)
+    cfg, tensors, model = build(dev, "float32", seed=seed, **_random_shape(rng))
+    g = torch.Generator().manual_seed(seed)
+    reqs = {"r%d" % i: torch.randint(0, cfg.vocab, (n,), generator=g).tolist()
+            for i, n in enumerate(rng.sample([5, 40, 90, 150, 230], 5))}
+    want = {k: oracle(cfg, tensors, v) for k, v in reqs.items()}
+    eng = engine(model, max_tokens=1024, seqs=4, blocks=34 + 1)  # 16-token pages: 1 + 3 + 6 + 10 + 15 would be 35
+    pending, live, at, got = list(reqs), [], {}, {k: [] for k in reqs}
+    while pending or live:
+        while pending and len(live) < 4 and (not live or rng.random() < 0.5):
+            live.append(pending.pop(0))
+            at[live[-1]] = 0
+        entries, end = [], []
+        for k in list(live):
+            if rng.random() < 0.15 and len(live) > 1:
+                continue  # left out of this step
+            n = min(len(reqs[k]) - at[k], rng.choice([1, 1, 1, 2, 3, 16, 37, 64, 150]))
+            entries.append((k, reqs[k][at[k]:at[k] + n], list(range(n))))
+            at[k] += n
+            if at[k] == len(reqs[k]):
+                live.remove(k)
+                end.append(k)
+        if not entries:
+            continue
+        out = eng.replay_step(entries, end)
+        r = 0
+        for k, tk, _ in entries:
+            got[k].append(out[r:r + len(tk)])
+            r += len(tk)
+    for k in reqs:
+        close(torch.cat(got[k]), want[k], 2e-4)
+    assert eng.bm.num_free == eng.bm.num_blocks - 1 and len(eng.state_slots.free) == 4
+
+
 # ------------------------------------------------------------------------------------------------ serving path
 @pytest.mark.parametrize("dev,dt", [("cpu", "float32"), pytest.param("cuda", "float32", marks=pytest.mark.gpu)])
 @pytest.mark.parametrize("native", [False, True])
