@@ -218,13 +218,17 @@ class HybridCache:
     * `tails[i]`: fp32 [state_slots, taps - 1, channels] last inputs of the run's causal convolution, or None.
 
     `spec` lists per run a dict with the optional keys "kv": (key row, value row), "state": (heads, P, N),
-    "tails": (taps - 1, channels). State slots are handed out per live sequence by `SlotPool`."""
+    "tails": (taps - 1, channels). State slots are handed out per live sequence by `SlotPool`. With `seq_tokens` the
+    cache also carries `last_token` int32 [state_slots]: the newest token of each live sequence, for embeddings that
+    look at the token before."""
 
-    def __init__(self, spec, num_blocks: int, block_size: int, device, dtype=torch.bfloat16, state_slots: int = 0):
+    def __init__(self, spec, num_blocks: int, block_size: int, device, dtype=torch.bfloat16, state_slots: int = 0,
+                 seq_tokens: bool = False):
         self.n_layers, self.num_blocks, self.block_size = len(spec), num_blocks, block_size
         self.state_slots = state_slots
         S = max(1, state_slots)
         f32 = dict(dtype=torch.float32, device=device)
+        self.last_token = torch.zeros(S, dtype=torch.int32, device=device) if seq_tokens else None
         self.kv, self.state, self.tails = [], [], []
         for e in spec:
             kv, st, tl = e.get("kv"), e.get("state"), e.get("tails")

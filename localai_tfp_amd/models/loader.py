@@ -152,16 +152,17 @@ def _state_families():
     """Decoder families served from a paged pool plus per-sequence state slots, chosen by config.json's
     `architecture`: name -> (module, model class name, config maker for `synthetic:<key>`)."""
     from . import girulorn as GI
+    from . import keronex as KE
     from . import vosotar as VO
     from . import vugotar as VU
     return {"vosotar": (VO, VO.VosotarModel, VO.is_vosotar_dir), "vugotar": (VU, VU.VugotarModel, VU.is_vugotar_dir),
-            "girulorn": (GI, GI.GirulornModel, GI.is_girulorn_dir)}
+            "girulorn": (GI, GI.GirulornModel, GI.is_girulorn_dir), "keronex": (KE, KE.KeronexModel, KE.is_keronex_dir)}
 
 
 def _load_latent(model: str, device, tp_size: int, ov: dict):
     """Latent-attention decoders (models/vosotar.py) and hybrid attention / recurrent decoders (models/vugotar.py,
-    models/girulorn.py): a directory whose config.json names the architecture, or `synthetic:vosotar-*` /
-    `synthetic:vugotar-*` / `synthetic:girulorn-*` random weights. `overrides["dtype"]`: torch.bfloat16 (default on GPU) | torch.float32. None for everything else."""
+    models/girulorn.py, models/keronex.py): a directory whose config.json names the architecture, or
+    `synthetic:vosotar-*` / `synthetic:vugotar-*` / `synthetic:girulorn-*` / `synthetic:keronex-*` random weights. `overrides["dtype"]`: torch.bfloat16 (default on GPU) | torch.float32. None for everything else."""
     from ..tokenizer import ByteTokenizer
     fam = None
     for key, (mod, klass, is_dir) in _state_families().items():

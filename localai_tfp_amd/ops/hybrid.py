@@ -21,7 +21,14 @@
 * `glu`: silu(a + bias) * (b + bias) with an optional per-row, per-column-group factor (routing weights of experts
   evaluated side by side, or the sigmoid gate of a shared expert);
 * `moe_route`: softmax over experts (optional logit bias), the `top` largest, renormalised and scaled, as a dense
-  [T, E] weight matrix (with eps = 0 and scale = 1 that is the softmax over the chosen logits alone).
+  [T, E] weight matrix (with eps = 0 and scale = 1 that is the softmax over the chosen logits alone); or, in the
+  `sigmoid` mode, the chosen experts' sigmoid scores as they are;
+* `embed_pair`: a scaled token embedding plus a row of a second table picked by a hash of (previous token, token); the
+  previous token is carried per sequence;
+* `hyper_step`: a residual kept as several streams: the streams are mixed among themselves and take a sublayer's
+  output with one weight each, and the next sublayer's input is a weighted sum of the streams, normed;
+* `rope_rows`: rotary positions in place, on neighbouring pairs or on the pairs (i, i + rot_dims / 2);
+* `diff_group_norm`: unit-RMS norm over groups of columns of a - lam * b (two attention maps over the same values).
 
 Every function runs the HIP kernels of csrc/kernels/hybrid/ on GPU tensors and a plain fp32 PyTorch form on CPU
 tensors (the plumbing path of GPU-less environments). Positions, angles, scores, softmax, norms, routing, decays,
@@ -105,6 +112,92 @@ def norm_add(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor, out1
     return x
 
 
+def embed_pair(table: torch.Tensor, pair: torch.Tensor | None, tokens: torch.Tensor, rag: "Ragged",
+               last_token: torch.Tensor | None, scale: float, mul_prev: int, mul_cur: int, buckets: int,
+               out: torch.Tensor, copies: int = 1):
+    """out[t] = scale * table[tokens[t]] + pair[(prev_t * mul_prev + tokens[t] * mul_cur) mod buckets], written
+    `copies` times side by side (out fp32 [T, copies * C]). prev_t is the token before row t in its sequence: the row
+    above inside a chunk, `last_token[slot]` (int32 [slots]) for a chunk's first row, and for position 0 there is none:
+    that row takes pair[buckets], the table's last row. Each sequence's last token of the step is left in
+    `last_token[slot]`. pair = None: the scaled embedding alone. Tables are fp32 or bf16."""
+    T = tokens.numel()
+    C = table.shape[1]
+    if T == 0:
+        return out
+    if out.shape != (T, copies * C) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError("embed_pair: out is a contiguous fp32 [T, copies * C]")
+    if pair is not None and (pair.shape != (buckets + 1, C) or last_token is None or last_token.dtype != torch.int32):
+        raise ValueError("embed_pair: the pair table has buckets + 1 rows; previous tokens are int32 per slot")
+    if not out.is_cuda:
+        tk = tokens.long()
+        x = table[tk].float() * scale
+        if pair is not None:
+            st, pos = rag.state.tolist(), rag.positions.tolist()
+            for r0, n, si in rag.host_segments():
+                slot = st[si]
+                prev = torch.empty(n, dtype=torch.long)
+                prev[1:] = tk[r0:r0 + n - 1]
+                first_none = pos[r0] == 0
+                prev[0] = 0 if (first_none or slot < 0) else int(last_token[slot])
+                row = (prev * mul_prev + tk[r0:r0 + n] * mul_cur) % buckets
+                if first_none:
+                    row[0] = buckets
+                x[r0:r0 + n] += pair[row].float()
+                if slot >= 0:
+                    last_token[slot] = int(tk[r0 + n - 1])
+        out.copy_(x.repeat(1, copies))
+        return out
+    if pair is not None and _is16(pair) != _is16(table):
+        raise TypeError("embed_pair: both tables share one dtype")
+    N.kcall("mxh_embed_pair", table.data_ptr(), N.ptr(pair), _is16(table), table.shape[0], tokens.data_ptr(),
+            rag.state.data_ptr(), rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, N.ptr(last_token),
+            float(scale), int(mul_prev), int(mul_cur), int(buckets), out.data_ptr(), int(copies), T, C, N.stream_ptr())
+    return out
+
+
+HYPER_MAX_STREAMS = 8
+
+
+def hyper_step(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, out_w: torch.Tensor | None,
+               in_w: torch.Tensor | None, norm_w: torch.Tensor | None, eps: float, h32: torch.Tensor | None = None,
+               h16: torch.Tensor | None = None, total: torch.Tensor | None = None, offset: float = 1.0):
+    """A residual of S streams xs fp32 [T, S * C] (stream s of a row in columns [s C, (s + 1) C)). With y (fp32 [T, C],
+    a sublayer's output): all streams at once from the old ones, x_t <- sum_s mix[s, t] x_s + out_w[t] y (mix fp32
+    [S, S] indexed [from, to], out_w fp32 [S]). With in_w (fp32 [S]): u = sum_s in_w[s] x_s of the updated streams and
+    h = u / sqrt(mean(u^2) + eps) * (offset + norm_w), written as fp32 (`h32`) and / or bf16 (`h16`): the input of the
+    next sublayer. `total` (fp32 [T, C]) receives the sum of the updated streams. One pass over the row."""
+    T = xs.shape[0]
+    if T == 0:
+        return
+    C = (y if y is not None else h32 if h32 is not None else h16 if h16 is not None else total).shape[1]
+    S = xs.shape[1] // C
+    if xs.shape[1] != S * C or S < 1 or S > HYPER_MAX_STREAMS:
+        raise ValueError(f"hyper_step: 1 to {HYPER_MAX_STREAMS} streams of one width")
+    if (y is None) != (mix is None) or (y is None) != (out_w is None) or (in_w is None) != (norm_w is None):
+        raise ValueError("hyper_step: an update needs y, mix and out_w; a read needs in_w and norm_w")
+    if not xs.is_cuda:
+        X = xs.view(T, S, C)
+        if y is not None:
+            X.copy_(torch.einsum("st,nsc->ntc", mix.float(), X) + out_w.float()[None, :, None] * y.float()[:, None, :])
+        if in_w is not None:
+            u = torch.einsum("s,nsc->nc", in_w.float(), X)
+            h = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * (offset + norm_w.float())
+            if h32 is not None:
+                h32.copy_(h)
+            if h16 is not None:
+                h16.copy_(h)
+        if total is not None:
+            total.copy_(X.sum(1))
+        return
+    _f32c(xs, "hyper_step")
+    if not xs.is_contiguous() or (y is not None and (y.dtype != torch.float32 or y.stride(1) != 1)):
+        raise TypeError("hyper_step: contiguous fp32 streams, fp32 rows of y")
+    N.kcall("mxh_hyper_step", xs.data_ptr(), N.ptr(y), y.stride(0) if y is not None else 0, N.ptr(mix), N.ptr(out_w),
+            N.ptr(in_w), N.ptr(norm_w), float(offset), float(eps), N.ptr(h32), h32.stride(0) if h32 is not None else 0,
+            N.ptr(h16), h16.stride(0) if h16 is not None else 0, N.ptr(total),
+            total.stride(0) if total is not None else 0, T, S, C, N.stream_ptr())
+
+
 # ------------------------------------------------------------------------------------------------ attention
 def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
     """Expands a bucketed distance-bias table rel [B, H] into one entry per distance and head: out [H, ceil(far) + 1]
@@ -126,9 +219,11 @@ def log_bucket_table(rel: torch.Tensor, far: float) -> torch.Tensor:
 def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor, positions: torch.Tensor, H: int,
                      G: int, dk: int, dv: int, rot_dims: int, rot_base: float, norm: bool, eps: float,
                      q_out: torch.Tensor, kc: torch.Tensor | None, vc: torch.Tensor | None, slots: torch.Tensor,
-                     q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, q_temp=None):
-    """q_in [T, H*dk], k_in [T, G*dk], v_in [T, G*dv]: fp32 column slices of one projection output. Pair (2i, 2i+1)
-    of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with `norm` every query
+                     q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, q_temp=None,
+                     half: bool = False, v_heads: int | None = None):
+    """q_in [T, H*dk], k_in [T, G*dk], v_in [T, Gv*dv] (Gv = v_heads, G when not given: the value pool may hold fewer
+    heads than the key pool): fp32 column slices of one projection output. Pair (2i, 2i+1), or with `half` the pair
+    (i, i + rot_dims/2), of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with `norm` every query
     and key head is then divided by its root mean square (eps inside the root) and multiplied by q_weight / k_weight
     (fp32 [dk], shared by the heads) when given. `q_temp` = (coef, every) multiplies the query at position p by
     1 + coef * ln(floor((p + 1) / every) + 1). Queries go to q_out [T, H*dk] (fp32 or bf16), keys and values into the
@@ -139,18 +234,10 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
         return
     if rot_dims % 2 or rot_dims > dk:
         raise ValueError("rope_norm_append: rot_dims is even and at most the head size")
+    Gv = G if v_heads is None else int(v_heads)
     if not q_in.is_cuda:
-        pos = positions.float()
-
         def turn(x, n, w=None):
-            x = x.float().reshape(T, n, dk).clone()
-            if rot_dims:
-                i = torch.arange(rot_dims // 2, dtype=torch.float32)
-                a = pos[:, None] * torch.exp(i * (-2.0 / rot_dims * math.log(rot_base)))[None, :]
-                c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
-                u, v = x[..., 0:rot_dims:2].clone(), x[..., 1:rot_dims:2].clone()
-                x[..., 0:rot_dims:2] = u * c - v * s
-                x[..., 1:rot_dims:2] = v * c + u * s
+            x = _rope_ref(x.float().reshape(T, n, dk), positions, rot_dims, rot_base, half)
             if norm:
                 x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
                 if w is not None:
@@ -165,14 +252,14 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
             return
         ok = slots >= 0
         kc.view(-1, G * dk)[slots[ok].long()] = turn(k_in, G, k_weight)[ok].to(kc.dtype)
-        vc.view(-1, G * dv)[slots[ok].long()] = v_in.float()[ok].to(vc.dtype)
+        vc.view(-1, Gv * dv)[slots[ok].long()] = v_in.float()[ok].to(vc.dtype)
         return
     if (q_weight is not None or k_weight is not None) and not norm:
         raise ValueError("rope_norm_append: head weights belong to the head norm")
     if k_in is None:  # queries only: no key / value heads in the grid
         k_in = v_in = q_in
         kc = vc = q_out
-        G = 0
+        G = Gv = 0
     else:
         if kc.dtype != vc.dtype or not kc.is_contiguous() or not vc.is_contiguous():
             raise TypeError("rope_norm_append: contiguous key and value pools of one dtype")
@@ -184,15 +271,58 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
     N.kcall("mxh_rope_norm_append", q_in.data_ptr(), k_in.data_ptr(), v_in.data_ptr(), q_in.stride(0),
             k_in.stride(0), v_in.stride(0), positions.data_ptr(), H, G, dk, dv, rot_dims, float(rot_base), int(norm),
             float(eps), q_out.data_ptr(), q_out.stride(0), _is16(q_out), kc.data_ptr(), vc.data_ptr(), _is16(kc),
-            slots.data_ptr(), N.ptr(q_weight), N.ptr(k_weight), coef, every, T, N.stream_ptr())
+            slots.data_ptr(), N.ptr(q_weight), N.ptr(k_weight), coef, every, int(half), Gv, T, N.stream_ptr())
+
+
+def _rope_ref(x: torch.Tensor, positions: torch.Tensor, rot_dims: int, rot_base: float, half: bool) -> torch.Tensor:
+    """x fp32 [T, n, d]: a copy whose first rot_dims numbers per head are turned by the rows' positions."""
+    x = x.clone()
+    if rot_dims:
+        n2 = rot_dims // 2
+        i = torch.arange(n2, dtype=torch.float32)
+        a = positions.float()[:, None] * torch.exp(i * (-2.0 / rot_dims * math.log(rot_base)))[None, :]
+        c, s = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+        lo, hi = (slice(0, n2), slice(n2, rot_dims)) if half else (slice(0, rot_dims, 2), slice(1, rot_dims, 2))
+        u, v = x[..., lo].clone(), x[..., hi].clone()
+        x[..., lo] = u * c - v * s
+        x[..., hi] = v * c + u * s
+    return x
+
+
+def rope_rows(x: torch.Tensor, positions: torch.Tensor, heads: int, dim: int, rot_dims: int, rot_base: float,
+              half: bool = False, scale: float = 1.0, split: int | None = None, scale2: float = 1.0):
+    """In place on fp32 x [T, heads*dim] (may be a column slice): rotary positions on the first rot_dims numbers of
+    every head (pairs as in `rope_norm_append`), then the head times `scale`; heads from index `split` on take
+    `scale2` (queries and keys side by side in one launch). For mixers that keep no keys per token."""
+    T = x.shape[0]
+    if T == 0:
+        return x
+    if rot_dims % 2 or rot_dims > dim:
+        raise ValueError("rope_rows: rot_dims is even and at most the head size")
+    split = heads if split is None else split
+    if not x.is_cuda:
+        v = _rope_ref(x.float().reshape(T, heads, dim), positions, rot_dims, rot_base, half)
+        sc = torch.full((heads, 1), float(scale))
+        sc[split:] = scale2
+        x.copy_((v * sc).reshape(T, heads * dim))
+        return x
+    _f32c(x, "rope_rows")
+    if dim > 512:
+        raise ValueError("rope_rows: heads of up to 512 numbers")
+    N.kcall("mxh_rope_rows", x.data_ptr(), x.stride(0), positions.data_ptr(), heads, dim, rot_dims, float(rot_base),
+            int(half), float(scale), int(split), float(scale2), T, N.stream_ptr())
+    return x
 
 
 def _attn_ref(q, kc, vc, table, ctx, pos0, H, G, dk, dv, scale, chunk, window, sink, out, out_scale, sink_v=None,
-              bias=None, gate=None):
+              bias=None, gate=None, Gv=None):
     bs = kc.shape[1]
     nb = -(-ctx // bs)
     k = kc[table[:nb].long()].reshape(nb * bs, G, dk)[:ctx].float()
-    v = vc[table[:nb].long()].reshape(nb * bs, G, dv)[:ctx].float()
+    Gv = G if Gv is None else Gv
+    v = vc[table[:nb].long()].reshape(nb * bs, Gv, dv)[:ctx].float()
+    if Gv != G:  # key head g reads value head g % Gv
+        v = v[:, torch.arange(G) % Gv]
     n = q.shape[0]
     qh = q.float().reshape(n, H, dk)
     rep = H // G
@@ -250,9 +380,11 @@ def _visible_blocks(p0: int, n: int, chunk: int, window: int, heads: int):
 
 
 def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window, sink, out, out_scale, sink_v=None,
-                     bias=None, gate=None):
+                     bias=None, gate=None, Gv=None, p32=False):
     """A long prompt chunk (rows q [n, H*dk] at positions p0 ..) as library GEMMs: per block of rows, the visible keys
-    and values are gathered head-major from the pages, scores = Q K^T (fp32), masked sink softmax, out = P V (fp32)."""
+    and values are gathered head-major from the pages, scores = Q K^T (fp32), masked sink softmax, out = P V (fp32).
+    With `p32` and bf16 operands every softmax weight is written as two bf16 numbers (its rounding and the rest), side
+    by side along K, and the values are stacked twice: the product sees the weights to 16 bits of mantissa."""
     from .dense import bmm_f32
     st = N.stream_ptr()
     md, dev, rep, bs = q.dtype, q.device, H // G, kc.shape[1]
@@ -262,17 +394,18 @@ def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window
         kh = torch.empty((G, nk, dk), dtype=md, device=dev)
         vh = torch.empty((G, nk, dv), dtype=md, device=dev)
         N.kcall("mxh_kv_gather", kc.data_ptr(), vc.data_ptr(), i16, bs, table.data_ptr(), key0, nk, G, dk, dv,
-                kh.data_ptr(), vh.data_ptr(), st)
+                kh.data_ptr(), vh.data_ptr(), G if Gv is None else Gv, st)
         qh = torch.empty((H, n2, dk), dtype=md, device=dev)
         qr = q[a - p0:]
         N.kcall("mxh_head_transpose", qr.data_ptr(), i16, qr.stride(0), dk, qh.data_ptr(), i16, dk, n2 * dk, n2, H, dk,
                 1.0, None, 0, st)
         sc = bmm_f32(qh.view(G, rep * n2, dk), kh.transpose(1, 2))
-        pw = torch.empty((G, rep * n2, nk), dtype=md, device=dev)
+        two = bool(p32 and i16)
+        pw = torch.empty((G, rep * n2, 2 * nk if two else nk), dtype=md, device=dev)
         N.kcall("mxh_masked_softmax", sc.data_ptr(), pw.data_ptr(), i16, H * n2, n2, nk, a, key0, float(scale),
                 int(chunk), int(window), int(sink), N.ptr(sink_v), N.ptr(bias), bias.shape[1] if bias is not None else 0,
-                H, st)
-        o = bmm_f32(pw, vh)
+                H, int(two), st)
+        o = bmm_f32(pw, torch.cat([vh, vh], 1) if two else vh)
         orow = out[a - p0:]
         grow = gate[a - p0:] if gate is not None else None
         N.kcall("mxh_head_transpose", o.data_ptr(), 0, dv, n2 * dv, orow.data_ptr(), _is16(out), orow.stride(0), dv, n2,
@@ -282,9 +415,12 @@ def _attn_gemm_chunk(q, kc, vc, table, p0, n, H, G, dk, dv, scale, chunk, window
 def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: Ragged, H: int, G: int, dk: int, dv: int,
                      scale: float, out: torch.Tensor, chunk: int = 0, window: int = 0, sink=False,
                      out_scale: float = 1.0, workspace=None, bias: torch.Tensor | None = None,
-                     gate: torch.Tensor | None = None):
-    """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key /
-    value head h // (H / G). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
+                     gate: torch.Tensor | None = None, v_heads: int | None = None, p32: bool = False):
+    """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key
+    head g = h // (H / G) and value head g % v_heads (v_heads = G when not given; fewer value heads than key heads:
+    several attention maps over the same values). `p32`: softmax weights enter the value product with more than
+    bf16's mantissa also in bf16 mode (the row kernels always do; the matrix-core kernels are left out, the GEMM
+    route splits each weight into two bf16 numbers). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
     max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
     [H] adds exp(sink[h]). `bias` (fp32 [H, L], contiguous) adds bias[h, min(i - j, L - 1)] to the scaled score.
     `gate` (fp32 [T, H], may be a column slice) multiplies head h's output of row t by sigmoid(gate[t, h]). out
@@ -301,6 +437,9 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
         return out
     if H % G:
         raise ValueError("masked_attention: heads must be a multiple of kv heads")
+    Gv = G if v_heads is None else int(v_heads)
+    if Gv < 1 or G % Gv:
+        raise ValueError("masked_attention: the key heads are a multiple of the value heads")
     sink_v = sink if isinstance(sink, torch.Tensor) else None
     sink = sink_v is not None or bool(sink)
     if sink_v is not None and (sink_v.dtype != torch.float32 or sink_v.numel() != H or not sink_v.is_contiguous()):
@@ -316,7 +455,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             lens = rag.dec_lens.tolist()
             for i in range(nd):
                 _attn_ref(q[i:i + 1], kc, vc, rag.dec_bt[i], lens[i], lens[i] - 1, H, G, dk, dv, scale, chunk, window,
-                          sink, out[i:i + 1], out_scale, sink_v, bias, gate[i:i + 1] if gate is not None else None)
+                          sink, out[i:i + 1], out_scale, sink_v, bias, gate[i:i + 1] if gate is not None else None, Gv)
         if rag.n_pf:
             cu, ctx = rag.pf_cu.tolist(), rag.pf_ctx.tolist()
             for k in range(rag.n_pf):
@@ -325,7 +464,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     r0 = nd + cu[k]
                     _attn_ref(q[r0:r0 + n], kc, vc, rag.pf_bt[k], ctx[k], ctx[k] - n, H, G, dk, dv, scale, chunk,
                               window, sink, out[r0:r0 + n], out_scale, sink_v, bias,
-                              gate[r0:r0 + n] if gate is not None else None)
+                              gate[r0:r0 + n] if gate is not None else None, Gv)
         return out
     if q.dtype != kc.dtype or kc.dtype != vc.dtype or q.stride(1) != 1 or out.stride(1) != 1:
         raise TypeError("masked_attention: queries and pools share one dtype, rows are contiguous")
@@ -335,7 +474,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     nb = bias.shape[1] if bias is not None else 0
     ldg = gate.stride(0) if gate is not None else 0
     extra = (N.ptr(sink_v), N.ptr(bias), nb)  # the gate pointer moves with the rows a launch serves
-    mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
+    mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and not p32 and \
         bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
     if nd:
         vis = rag.dec_max_len
@@ -355,12 +494,12 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), rag.dec_lens.data_ptr(), nd, out.data_ptr(),
                     out.stride(0), _is16(out), H, G, dk, dv, float(scale), int(chunk), int(window), int(sink),
                     float(out_scale), parts, plen if parts > 1 else 0, N.ptr(ml), N.ptr(po), *extra, N.ptr(gate), ldg,
-                    st)
+                    Gv, st)
         else:
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
                     out.data_ptr(), out.stride(0), _is16(out), *common, 0, parts, plen if parts > 1 else 0, N.ptr(ml),
-                    N.ptr(po), *extra, N.ptr(gate), ldg, st)
+                    N.ptr(po), *extra, N.ptr(gate), ldg, Gv, st)
     if rag.n_pf:
         lens = rag.pf_q_host if len(rag.pf_q_host) == rag.n_pf and len(rag.pf_ctx_host) == rag.n_pf else None
 
@@ -368,7 +507,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.pf_bt.data_ptr(), rag.pf_bt.stride(0), rag.pf_cu.data_ptr(), rag.pf_ctx.data_ptr(), rag.n_pf,
                     n_rows, nd, out.data_ptr(), out.stride(0), _is16(out), *common, row_off, 1, 0, None, None, *extra,
-                    N.ptr(gate), ldg, st)
+                    N.ptr(gate), ldg, Gv, st)
         mfma = mfma_ok
         big = MFMA_MIN_ROWS if mfma else GEMM_MIN_ROWS
         if lens is None or max(lens) < big or (not mfma and 0 < chunk < GEMM_MIN_ROWS):
@@ -386,10 +525,10 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     N.kcall("mxh_attention_mfma", qk.data_ptr(), qk.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
                             rag.pf_bt[k].data_ptr(), rag.pf_ctx_host[k] - n, n, ok.data_ptr(), ok.stride(0), _is16(out),
                             H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale), *extra,
-                            N.ptr(gk), ldg, st)
+                            N.ptr(gk), ldg, Gv, st)
                 else:
                     _attn_gemm_chunk(qk, kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv, scale, chunk,
-                                     window, sink, ok, out_scale, sink_v, bias, gk)
+                                     window, sink, ok, out_scale, sink_v, bias, gk, Gv, p32)
             elif n and run0 is None:
                 run0 = r
             r += n
@@ -475,9 +614,10 @@ def scan_coefs(a: torch.Tensor, b: torch.Tensor | None, A_log: torch.Tensor, dt_
 
 
 def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: torch.Tensor,
-                  proj: torch.Tensor | None = None):
+                  proj: torch.Tensor | None = None, rate_log: torch.Tensor | None = None):
     """out = sigmoid(x)^(1 / tau), computed as exp(log_sigmoid(x) / tau): the per-channel decay of gated linear
-    attention. x = z + bias with z fp32 [T, C]; or, with `proj` (fp32 [R, C], contiguous), x = z proj + bias with z
+    attention; or, with `rate_log` (fp32 [heads], C / heads channels per head, tau unused),
+    out = exp(-exp(rate_log[head]) * softplus(x)): a step size per channel under a learned rate per head. x = z + bias with z fp32 [T, C]; or, with `proj` (fp32 [R, C], contiguous), x = z proj + bias with z
     fp32 [T, R]: the second half of a low-rank projection, done in fp32 inside the same kernel. z may be a column
     slice; bias fp32 [C]; out fp32 [T, C] contiguous."""
     T, C = out.shape
@@ -489,27 +629,36 @@ def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: t
         x = z.float() @ proj.float() if proj is not None else z.float()
         if bias is not None:
             x = x + bias.float()
-        out.copy_(torch.exp(F.logsigmoid(x) / tau))
+        if rate_log is not None:
+            rate = torch.exp(rate_log.float()).repeat_interleave(C // rate_log.numel())
+            out.copy_(torch.exp(-rate * F.softplus(x, threshold=30.0)))
+        else:
+            out.copy_(torch.exp(F.logsigmoid(x) / tau))
         return out
     _f32c(z, "channel_decay")
+    if rate_log is not None and (rate_log.dtype != torch.float32 or C % rate_log.numel()):
+        raise ValueError("channel_decay: one fp32 rate per head, whole heads of channels")
     if not out.is_contiguous() or out.dtype != torch.float32 or tau <= 0:
         raise ValueError("channel_decay: contiguous fp32 output, tau > 0")
     if proj is not None and (proj.dtype != torch.float32 or not proj.is_contiguous()):
         raise TypeError("channel_decay: the projection is a contiguous fp32 [R, C] matrix")
     N.kcall("mxh_channel_decay", z.data_ptr(), z.stride(0), N.ptr(bias), float(1.0 / tau), out.data_ptr(), T, C,
-            N.ptr(proj), proj.shape[0] if proj is not None else 0, N.stream_ptr())
+            N.ptr(proj), proj.shape[0] if proj is not None else 0, N.ptr(rate_log),
+            C // rate_log.numel() if rate_log is not None else 0, N.stream_ptr())
     return out
 
 
 def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, coef: torch.Tensor | None,
                skip: torch.Tensor | None, state: torch.Tensor, rag: Ragged, out: torch.Tensor, H: int, G: int, Nk: int,
-               P: int, delta: bool, channel: bool = False, q_scale: float = 1.0):
+               P: int, delta: bool, channel: bool = False, q_scale: float = 1.0, coef_sigmoid: bool = False):
     """Linear recurrence per sequence and head over the step's rows, in order:
         S <- decay_t S;  u = coef_t (v_t - S^T k_t) if delta else coef_t v_t;  S <- S + k_t u^T;
         o_t = S^T (q_scale q_t) (+ skip_h v_t)
     k, q fp32 [T, G*Nk] (head h reads group h // (H / G)), v fp32 [T, H*P], decay / coef fp32 [T, H], out fp32
     [T, H*P]; all may be column slices. With `channel` the decay is fp32 [T, H*Nk], one number per head and key
-    channel (row n of S is multiplied by decay[h, n]: gated linear attention). coef = None means 1.
+    channel (row n of S is multiplied by decay[h, n]: gated linear attention, or with `delta` a delta rule with a decay
+    per key channel). A decay of shape [H] is one constant per head for every token (retention). coef = None means 1; with `coef_sigmoid` coef holds
+    pre-activations (a column slice of a projection's output) and the write strength is their sigmoid.
     state fp32 [slots, H, P, Nk] (a column's Nk numbers are contiguous) is read at
     the sequence's slot unless its first row is at position 0 (then S starts at zero) and written back after its last
     row."""
@@ -526,8 +675,9 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
                 kt = k[t].float().reshape(G, Nk).repeat_interleave(rep, 0)
                 qt = q[t].float().reshape(G, Nk).repeat_interleave(rep, 0) * q_scale
                 vt = v[t].float().reshape(H, P)
-                S = S * (decay[t].reshape(H, Nk)[:, :, None] if channel else decay[t][:, None, None])
-                cf = coef[t][:, None] if coef is not None else 1.0
+                dt = decay if decay.dim() == 1 else decay[t]
+                S = S * (dt.reshape(H, Nk)[:, :, None] if channel else dt[:, None, None])
+                cf = (torch.sigmoid(coef[t].float()) if coef_sigmoid else coef[t])[:, None] if coef is not None else 1.0
                 u = cf * ((vt - torch.einsum("hnp,hn->hp", S, kt)) if delta else vt)
                 S = S + kt[:, :, None] * u[:, None, :]
                 o = torch.einsum("hnp,hn->hp", S, qt)
@@ -540,89 +690,161 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
     for t_ in (k, q, v, out):
         _f32c(t_, "state_scan")
     if tuple(state.shape[1:]) != (H, P, Nk) or not state.is_contiguous() or not decay.is_contiguous() \
-            or (coef is not None and not coef.is_contiguous()) or H % G or Nk > 256:
-        raise ValueError("state_scan: state is [slots, H, P, N] with N <= 256, decay / coef contiguous [T, H]")
-    if decay.shape[-1] != (H * Nk if channel else H) or (channel and delta):
-        raise ValueError("state_scan: one decay per head, or per head and key channel (not with the delta rule)")
+            or (coef is not None and (coef.stride(1) != 1 or coef.dtype != torch.float32)) or H % G or Nk > 256:
+        raise ValueError("state_scan: state is [slots, H, P, N] with N <= 256, decay contiguous, coef fp32 [T, H]")
+    if decay.shape[-1] != (H * Nk if channel else H) or (decay.dim() == 1 and channel) or decay.dtype != torch.float32:
+        raise ValueError("state_scan: one fp32 decay per head, or per head and key channel")
     N.kcall("mxh_state_scan", k.data_ptr(), k.stride(0), q.data_ptr(), q.stride(0), v.data_ptr(), v.stride(0),
-            decay.data_ptr(), N.ptr(coef), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
+            decay.data_ptr(), 0 if decay.dim() == 1 else 1, N.ptr(coef),
+            coef.stride(0) if coef is not None else 0, int(coef_sigmoid), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
             rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, out.data_ptr(), out.stride(0), H, G, Nk,
             P, int(delta), int(channel), float(q_scale), N.stream_ptr())
     return out
 
 
-def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float, group: int, out: torch.Tensor,
-                     gate_first: bool, out_scale: float = 1.0):
+def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor | None, eps: float, group: int,
+                     out: torch.Tensor, gate_first: bool, out_scale: float = 1.0, act: str = "silu",
+                     proj: torch.Tensor | None = None):
     """Rows y [T, C] fp32 in groups of `group` columns, gate [T, C] fp32 (pre-activation), w fp32 whose length divides
-    C (column c uses w[c % len(w)]). gate_first: z = y * silu(gate), out = unit_rms_group(z) * w; otherwise
-    out = unit_rms_group(y) * w * silu(gate). out (fp32 or bf16, may be a column slice) gets out_scale times that."""
+    C (column c uses w[c % len(w)]; None: no weight). gate_first: z = y * act(gate), out = unit_rms_group(z) * w;
+    otherwise out = unit_rms_group(y) * w * act(gate); act is "silu" or "sigmoid". With `proj` (fp32 [R, C], contiguous)
+    the gate is [T, R] and its pre-activation is gate proj, summed in fp32 inside the kernel (the second half of a
+    low-rank gate). out (fp32 or bf16, may be a column slice) gets out_scale times that."""
     T, C = y.shape
     if T == 0:
         return out
+    if act not in ("silu", "sigmoid"):
+        raise ValueError("gated_group_norm: the gate is a silu or a sigmoid")
+    if w is None:
+        w = _ones(y.device)
     if C % group or C % w.numel():
         raise ValueError("gated_group_norm: group size and weight length divide the row")
+    if gate.shape != ((T, proj.shape[0]) if proj is not None else (T, C)) or (proj is not None and proj.shape[1] != C):
+        raise ValueError("gated_group_norm: the gate is [T, C], or [T, R] beside a projection [R, C]")
     if not y.is_cuda:
-        g = F.silu(gate.float())
+        gp = gate.float() @ proj.float() if proj is not None else gate.float()
+        g = F.silu(gp) if act == "silu" else torch.sigmoid(gp)
         z = (y.float() * g if gate_first else y.float()).reshape(T, C // group, group)
         z = (z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, C) * w.float().repeat(C // w.numel())
         out.copy_(((z if gate_first else z * g) * out_scale).to(out.dtype))
         return out
     _f32c(y, "gated_group_norm")
     _f32c(gate, "gated_group_norm")
+    if proj is not None and (proj.dtype != torch.float32 or not proj.is_contiguous()):
+        raise TypeError("gated_group_norm: the projection is a contiguous fp32 [R, C] matrix")
     N.kcall("mxh_gated_group_norm", y.data_ptr(), y.stride(0), gate.data_ptr(), gate.stride(0), w.data_ptr(),
             w.numel(), float(eps), group, int(gate_first), float(out_scale), out.data_ptr(), out.stride(0), _is16(out),
-            T, C, N.stream_ptr())
+            T, C, int(act == "sigmoid"), N.ptr(proj), proj.shape[0] if proj is not None else 0, N.stream_ptr())
+    return out
+
+
+_ONES: dict = {}
+
+
+def _ones(device) -> torch.Tensor:
+    """A one-element fp32 tensor holding 1 (the weight of a norm without weights)."""
+    t = _ONES.get(device)
+    if t is None:
+        t = _ONES[device] = torch.ones(1, dtype=torch.float32, device=device)
+    return t
+
+
+def diff_group_norm(a: torch.Tensor, b: torch.Tensor, lam: float, eps: float, group: int, out: torch.Tensor,
+                    out_scale: float = 1.0):
+    """out = unit_rms_group(a - lam * b) * out_scale over groups of `group` columns: two attention maps over the same
+    values combined per head (differential attention) and normed without a weight. a, b fp32 [T, C] (column slices
+    allowed), out fp32 or bf16 [T, C] (may be a column slice)."""
+    T, C = a.shape
+    if T == 0:
+        return out
+    if C % group or b.shape != a.shape:
+        raise ValueError("diff_group_norm: two [T, C] inputs, whole groups")
+    if not a.is_cuda:
+        z = (a.float() - lam * b.float()).reshape(T, C // group, group)
+        z = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+        out.copy_(z.reshape(T, C).to(out.dtype))
+        return out
+    _f32c(a, "diff_group_norm")
+    _f32c(b, "diff_group_norm")
+    if group > 8192:
+        raise ValueError("diff_group_norm: groups of up to 8192 numbers")
+    N.kcall("mxh_diff_group_norm", a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), float(lam), float(eps), group,
+            float(out_scale), out.data_ptr(), out.stride(0), _is16(out), T, C, N.stream_ptr())
     return out
 
 
 # ------------------------------------------------------------------------------------------------ feed-forward
-def glu(a: torch.Tensor, b: torch.Tensor, bias_a: torch.Tensor | None, bias_b: torch.Tensor | None, out: torch.Tensor,
-        scale: torch.Tensor | None = None, group: int = 0, scale_sigmoid: bool = False):
-    """out = silu(a + bias_a) * (b + bias_b) [* factor]; a, b fp32 [T, F] column slices, out fp32 or bf16 [T, F] (may
-    be a column slice). `scale` fp32 [T, F / group] (column slice allowed) gives one factor per row and group of
-    `group` columns, passed through a sigmoid first with `scale_sigmoid`."""
+GLU_ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}
+
+
+def glu(a: torch.Tensor, b: torch.Tensor | None, bias_a: torch.Tensor | None, bias_b: torch.Tensor | None,
+        out: torch.Tensor, scale: torch.Tensor | None = None, group: int = 0, scale_sigmoid: bool = False,
+        act: str = "silu"):
+    """out = act(a + bias_a) * (b + bias_b) [* factor] with act "silu" or "gelu_tanh" (0.5 z (1 + tanh(sqrt(2 / pi)
+    (z + 0.044715 z^3)))); a, b fp32 [T, F] column slices, out fp32 or bf16 [T, F] (may be a column slice). `scale`
+    fp32 [T, F / group] (column slice allowed) gives one factor per row and group of `group` columns, passed through a
+    sigmoid first with `scale_sigmoid`. act "relu2" has no second operand (b = None) and the factor multiplies the
+    INPUT: out = relu(factor * (a + bias_a))^2, an expert that is fed its routing weight times the token."""
     T, Fn = a.shape
     if T == 0 or Fn == 0:
         return out
+    if act not in GLU_ACTS or (b is None) != (act == "relu2"):
+        raise ValueError("glu: act is silu | gelu_tanh with two operands, or relu2 with one")
     if not a.is_cuda:
         x = a.float() + bias_a if bias_a is not None else a.float()
-        y = b.float() + bias_b if bias_b is not None else b.float()
-        z = F.silu(x) * y
+        s = None
         if scale is not None:
             s = torch.sigmoid(scale.float()) if scale_sigmoid else scale.float()
-            z = (z.reshape(T, Fn // group, group) * s[:, :, None]).reshape(T, Fn)
+            s = s.repeat_interleave(group, 1)
+        if act == "relu2":
+            z = torch.relu(x * s if s is not None else x).pow(2)
+        else:
+            y = b.float() + bias_b if bias_b is not None else b.float()
+            z = (F.silu(x) if act == "silu" else F.gelu(x, approximate="tanh")) * y
+            if s is not None:
+                z = z * s
         out.copy_(z.to(out.dtype))
         return out
     _f32c(a, "glu")
-    _f32c(b, "glu")
+    if b is not None:
+        _f32c(b, "glu")
     if scale is not None and (group <= 0 or Fn % group or scale.shape[1] != Fn // group):
         raise ValueError("glu: one factor per row and group of columns")
-    N.kcall("mxh_glu", a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), N.ptr(bias_a), N.ptr(bias_b),
-            N.ptr(scale), scale.stride(0) if scale is not None else 0, group if scale is not None else Fn,
-            int(scale_sigmoid), out.data_ptr(), out.stride(0), _is16(out), T, Fn, N.stream_ptr())
+    N.kcall("mxh_glu", a.data_ptr(), a.stride(0), N.ptr(b), b.stride(0) if b is not None else 0, N.ptr(bias_a),
+            N.ptr(bias_b), N.ptr(scale), scale.stride(0) if scale is not None else 0,
+            group if scale is not None else Fn, int(scale_sigmoid), out.data_ptr(), out.stride(0), _is16(out), T, Fn,
+            GLU_ACTS[act], N.stream_ptr())
     return out
 
 
 def moe_route(logits: torch.Tensor, top: int, scale: float, weights: torch.Tensor, eps: float = 1e-20,
-              bias: torch.Tensor | None = None):
+              bias: torch.Tensor | None = None, mode: str = "softmax"):
     """Router of a mixture of experts: s = softmax(logits + bias) over all E experts, the `top` largest are kept,
     divided by their sum (+ eps) and multiplied by `scale` (eps = 0, scale = 1: the softmax over the chosen logits
     alone). logits fp32 [T, E] (column slice allowed), bias fp32 [E]; weights fp32 [T, E] contiguous: the chosen
-    experts' weights, 0 elsewhere. Ties go to the lower expert index."""
+    experts' weights, 0 elsewhere. Ties go to the lower expert index. mode "sigmoid": the scores are
+    sigmoid(logits + bias), the `top` largest are chosen and keep their scores as weights, times `scale`, not
+    renormalised."""
     T, E = logits.shape
     if T == 0:
         return weights
     if not 0 < top <= E:
         raise ValueError("moe_route: 1 <= top <= experts")
+    if mode not in ("softmax", "sigmoid"):
+        raise ValueError("moe_route: softmax or sigmoid scores")
     if not logits.is_cuda:
-        s = torch.softmax(logits.float() + bias.float() if bias is not None else logits.float(), -1)
-        tv, ti = torch.topk(s, top, dim=-1)
+        z = logits.float() + bias.float() if bias is not None else logits.float()
         weights.zero_()
+        if mode == "sigmoid":
+            tv, ti = torch.topk(z, top, dim=-1)
+            weights.scatter_(1, ti, torch.sigmoid(tv) * scale)
+            return weights
+        tv, ti = torch.topk(torch.softmax(z, -1), top, dim=-1)
         weights.scatter_(1, ti, tv / (tv.sum(-1, keepdim=True) + eps) * scale)
         return weights
     _f32c(logits, "moe_route")
     if E > 1024:
         raise ValueError("moe_route: at most 1024 experts")
     N.kcall("mxh_moe_route", logits.data_ptr(), logits.stride(0), N.ptr(bias), T, E, top, float(scale), float(eps),
-            weights.data_ptr(), N.stream_ptr())
+            weights.data_ptr(), int(mode == "sigmoid"), N.stream_ptr())
     return weights
