@@ -1,7 +1,8 @@
 // hybrid_attn.hip: causal softmax attention over paged key / value pools with a visible range that starts at a chunk
 // border, a window's edge or position 0, and an optional sink term in the denominator (ops/hybrid.py
 // masked_attention). Pools are token-major: keys [blocks, bs, G * dk], values [blocks, bs, G * dv], fp32 or bf16.
-// Every kernel also takes an AttnExtra: a learned sink score per head instead of 0, an additive bias looked up by the
+// The value pool may hold fewer heads than the key pool (gv of them, a divisor of G): key head g then reads value
+// head g % gv, several attention maps over the same values. Every kernel also takes an AttnExtra: a learned sink score per head instead of 0, an additive bias looked up by the
 // distance between query and key (table [H, distances], the last entry serving every larger distance), and a gate per
 // row and head whose sigmoid multiplies the head's output.
 //
@@ -31,6 +32,7 @@ struct AttnExtra {
     int nb;
     const float* gate;    // pre-sigmoid gate of row r and head h at gate[r * ldg + h] (null: none)
     int ldg;
+    int gv;               // value heads in the pool: key head g reads value head g % gv
 };
 MX_DEV float sink_score(const AttnExtra& ex, int h) { return ex.sink_v ? ex.sink_v[h] : 0.f; }
 MX_DEV float dist_bias(const AttnExtra& ex, int dist, int H, int h) {
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
         __syncthreads();  // the previous tile's weights and offsets have been read
 #pragma unroll
         for (int i = 0; i < REP; ++i) ps[i * 64 + lane] = p[i];
-        rowoff[lane] = (tok * G + g) * dv;
+        rowoff[lane] = (tok * ex.gv + g % ex.gv) * dv;
         __syncthreads();
         const int nk = min(64, pos - j0 + 1);
         // VB keys' values for all of the lane's columns are requested together (clamped columns: no branch between
@@ -261,8 +263,9 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const void* q, int ldq, c
 // array references: the pieces stay in registers.
 template <int DK, int DV, int KT, int NTH>
 MX_DEV void tile_load(u32x4 (&kr)[KT * DK / 8 / NTH], u32x4 (&vr)[KT * DV / 8 / NTH], const bf16_t* __restrict__ kc,
-                      const bf16_t* __restrict__ vc, const int* __restrict__ table, int bs, int G, int kvh, int kt0,
-                      int kv_end, int tid) {
+                      const bf16_t* __restrict__ vc, const int* __restrict__ table, int bs, int G, int kvh, int Gv,
+                      int kt0, int kv_end, int tid) {
+    const int vh = kvh % Gv;
 #pragma unroll
     for (int j = 0; j < KT * DK / 8 / NTH; ++j) {
         const int id = tid + j * NTH;
@@ -277,7 +280,7 @@ MX_DEV void tile_load(u32x4 (&kr)[KT * DK / 8 / NTH], u32x4 (&vr)[KT * DV / 8 / 
         const int p = id / (DV / 8), c = id % (DV / 8);
         const int pos = min(kt0 + p, kv_end - 1);
         const size_t tok = (size_t)table[pos / bs] * bs + (pos % bs);
-        vr[j] = *(const u32x4*)(vc + (tok * G + kvh) * DV + c * 8);
+        vr[j] = *(const u32x4*)(vc + (tok * Gv + vh) * DV + c * 8);
     }
 }
 template <int DK, int DV, int KT, int NTH, int KSTR, int VSTR>
@@ -373,7 +376,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
 
     constexpr int KCH = KT * DK / 8 / 256, VCH = KT * DV / 8 / 256;  // 16-byte pieces per thread
     u32x4 kr[KCH], vr[VCH];
-#define LOAD_TILE(kt0_) tile_load<DK, DV, KT, 256>(kr, vr, kc, vc, table, bs, G, kvh, kt0_, kv_end, threadIdx.x)
+#define LOAD_TILE(kt0_) tile_load<DK, DV, KT, 256>(kr, vr, kc, vc, table, bs, G, kvh, ex.gv, kt0_, kv_end, threadIdx.x)
 #define STORE_TILE() tile_store<DK, DV, KT, 256, KSTR, VSTR>(kr, vr, k_lds, v_lds, threadIdx.x)
     if (kt_begin < kv_end) LOAD_TILE(kt_begin);
     for (int kt0 = kt_begin; kt0 < kv_end; kt0 += KT) {
@@ -556,7 +559,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
             const int id = lane + j * 64;
             const int p = id / (DV / 8), c = id % (DV / 8);
             const int pos = min(kt0 + p, kv_end - 1);
-            vr[j] = *(const u32x4*)(vc + (((size_t)table[pos / bs] * bs + (pos % bs)) * G + kvh) * DV + c * 8);
+            vr[j] = *(const u32x4*)(vc + (((size_t)table[pos / bs] * bs + (pos % bs)) * ex.gv + kvh % ex.gv) * DV + c * 8);
         }
     };
     if (lo < kv_end) load_tile(lo);
@@ -708,15 +711,15 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* part_ml, co
 }
 
 // grid (keys, G): key jj of the range is the token at position lo + jj of the sequence whose block table is `table`;
-// its group's key and value rows go to kh [G][n][dk] and vh [G][n][dv]
+// its group's key and value rows go to kh [G][n][dk] and vh [G][n][dv] (the value row of head g % Gv)
 template <typename E>
 __global__ __launch_bounds__(64) void kv_gather_kernel(const E* kc, const E* vc, int bs, const int* table, int lo, int n,
-                                                       int G, int dk, int dv, E* kh, E* vh) {
+                                                       int G, int dk, int dv, E* kh, E* vh, int Gv) {
     const int jj = blockIdx.x, g = blockIdx.y;
     const int j = lo + jj;
     const long tok = (long)table[j / bs] * bs + (j % bs);
     const E* ks = kc + (tok * G + g) * dk;
-    const E* vs = vc + (tok * G + g) * dv;
+    const E* vs = vc + (tok * Gv + g % Gv) * dv;
     E* kd = kh + ((long)g * n + jj) * dk;
     E* vd = vh + ((long)g * n + jj) * dv;
     for (int e = threadIdx.x; e < dk; e += 64) kd[e] = ks[e];
@@ -737,11 +740,14 @@ __global__ __launch_bounds__(64) void head_transpose_kernel(const void* src, lon
 }
 
 // grid (H * n): row (h, i) holds the raw scores of the query at position p0 + i against the keys at positions
-// key0 .. key0 + nk - 1. Writes the masked, sink-normalised softmax weights (zeros outside the visible range).
+// key0 .. key0 + nk - 1. Writes the masked, sink-normalised softmax weights (zeros outside the visible range). With
+// `two` (bf16 weights) a row of the output holds 2 nk numbers: every weight's bf16 rounding, then the bf16 roundings
+// of what the first rounding lost, so that a product with the values stacked twice sees 16 bits of each weight.
 template <bool P16>
 __global__ __launch_bounds__(256) void masked_softmax_kernel(const float* sc, void* pw, int n, int nk, int p0, int key0,
                                                              float scale, int chunk, int window, int sink,
-                                                             const float* sink_v, const float* bias, int nb, int H) {
+                                                             const float* sink_v, const float* bias, int nb, int H,
+                                                             int two) {
     __shared__ float red[4];
     const long row = blockIdx.x;
     const int i = (int)(row % n), h = (int)(row / n);
@@ -761,8 +767,17 @@ __global__ __launch_bounds__(256) void masked_softmax_kernel(const float* sc, vo
     const float inv = 1.f / l;
     for (int j = threadIdx.x; j < nk; j += 256) {
         const float p = (j >= a && j <= b) ? expf(score(j) - m) * inv : 0.f;
-        if constexpr (P16) ((bf16_t*)pw)[row * nk + j] = f32_to_bf16(p);
-        else ((float*)pw)[row * nk + j] = p;
+        if constexpr (P16) {
+            const bf16_t hi = f32_to_bf16(p);
+            if (two) {
+                ((bf16_t*)pw)[row * 2 * nk + j] = hi;
+                ((bf16_t*)pw)[row * 2 * nk + nk + j] = f32_to_bf16(p - bf16_to_f32(hi));
+            } else {
+                ((bf16_t*)pw)[row * nk + j] = hi;
+            }
+        } else {
+            ((float*)pw)[row * nk + j] = p;
+        }
     }
 }
 
@@ -776,10 +791,10 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
                              void* out, int ldo, int o16, int H, int G, int dk, int dv, float scale, int chunk,
                              int window, int sink, float out_scale, int row_off, int parts, int part_len,
                              float* part_ml, float* part_o, const float* sink_v, const float* bias, int nb,
-                             const float* gate, int ldg, hipStream_t st) {
+                             const float* gate, int ldg, int gv, hipStream_t st) {
     if (n_rows <= 0 || n_seqs <= 0) return 0;
-    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
-    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink) && gv > 0 && G % gv == 0);
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg, gv};
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0);
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && dk > 0 && dv > 0 && dv <= 64 * DVU_MAX && dk <= 4096);
     MXH_CHECK(ldq >= H * dk && ldo >= H * dv && chunk >= 0 && window >= 0 && H <= 65535 && row_off >= 0);
@@ -815,14 +830,15 @@ extern "C" int mxh_attention(const void* q, int ldq, int q16, const void* kc, co
 }
 
 extern "C" int mxh_kv_gather(const void* kc, const void* vc, int is16, int bs, const int* table, int lo, int n, int G,
-                             int dk, int dv, void* kh, void* vh, hipStream_t st) {
+                             int dk, int dv, void* kh, void* vh, int Gv, hipStream_t st) {
     if (n <= 0) return 0;
     MXH_CHECK(kc && vc && table && kh && vh && bs > 0 && lo >= 0 && G > 0 && G <= 65535 && dk > 0 && dv > 0);
+    MXH_CHECK(Gv > 0 && G % Gv == 0);
     const dim3 grid(n, G);
     if (is16) kv_gather_kernel<bf16_t><<<grid, 64, 0, st>>>((const bf16_t*)kc, (const bf16_t*)vc, bs, table, lo, n, G, dk,
-                                                           dv, (bf16_t*)kh, (bf16_t*)vh);
+                                                           dv, (bf16_t*)kh, (bf16_t*)vh, Gv);
     else kv_gather_kernel<float><<<grid, 64, 0, st>>>((const float*)kc, (const float*)vc, bs, table, lo, n, G, dk, dv,
-                                                      (float*)kh, (float*)vh);
+                                                      (float*)kh, (float*)vh, Gv);
     return (int)hipGetLastError();
 }
 
@@ -843,16 +859,17 @@ extern "C" int mxh_head_transpose(const void* src, int s16, long s_si, long s_sh
 
 extern "C" int mxh_masked_softmax(const float* sc, void* pw, int p16, long rows, int n, int nk, int p0, int key0,
                                   float scale, int chunk, int window, int sink, const float* sink_v,
-                                  const float* bias, int nb, int H, hipStream_t st) {
+                                  const float* bias, int nb, int H, int two, hipStream_t st) {
     if (rows <= 0) return 0;
+    MXH_CHECK(!two || p16);
     MXH_CHECK(sc && pw && n > 0 && nk > 0 && rows % n == 0 && rows < (1L << 31) && key0 >= 0 && p0 >= key0);
     MXH_CHECK((!bias || nb > 0) && (!(bias || sink_v) || rows == (long)H * n));
     if (p16)
         masked_softmax_kernel<true><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink,
-                                                                    sink_v, bias, nb, H);
+                                                                    sink_v, bias, nb, H, two);
     else
         masked_softmax_kernel<false><<<(unsigned)rows, 256, 0, st>>>(sc, pw, n, nk, p0, key0, scale, chunk, window, sink,
-                                                                     sink_v, bias, nb, H);
+                                                                     sink_v, bias, nb, H, 0);
     return (int)hipGetLastError();
 }
 
@@ -863,10 +880,10 @@ extern "C" int mxh_attention_mfma_ok(int dk, int dv) { return (dk == 64 || dk ==
 extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const void* vc, int bs, const int* table,
                                   int p0, int n, void* out, int ldo, int o16, int H, int G, int dk, int dv,
                                   float scale, int chunk, int window, int sink, float out_scale, const float* sink_v,
-                                  const float* bias, int nb, const float* gate, int ldg, hipStream_t st) {
+                                  const float* bias, int nb, const float* gate, int ldg, int gv, hipStream_t st) {
     if (n <= 0) return 0;
-    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
-    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink) && gv > 0 && G % gv == 0);
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg, gv};
     MXH_CHECK(q && kc && vc && table && out && bs > 0 && p0 >= 0 && H > 0 && G > 0 && H % G == 0);
     MXH_CHECK(mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv && chunk >= 0 && window >= 0);
     const int rep = H / G;
@@ -900,10 +917,10 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
                                          int G, int dk, int dv, float scale, int chunk, int window, int sink,
                                          float out_scale, int parts, int part_len, float* part_ml, float* part_o,
                                          const float* sink_v, const float* bias, int nb, const float* gate, int ldg,
-                                         hipStream_t st) {
+                                         int gv, hipStream_t st) {
     if (n_seqs <= 0) return 0;
-    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink));
-    const AttnExtra ex = {sink_v, bias, nb, gate, ldg};
+    MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink) && gv > 0 && G % gv == 0);
+    const AttnExtra ex = {sink_v, bias, nb, gate, ldg, gv};
     MXH_CHECK(q && kc && vc && bt && ctx && out && bs > 0 && bt_stride > 0 && H > 0 && G > 0 && H % G == 0);
     MXH_CHECK(H / G <= 16 && G <= 65535 && mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv);
     MXH_CHECK(parts >= 1 && parts <= 64 && (parts == 1 || (part_len > 0 && part_ml && part_o)) && chunk >= 0 && window >= 0);

@@ -151,8 +151,9 @@ __global__ __launch_bounds__(1024) void norm_add_kernel(const float* y, int ldy,
     }
 }
 
-// grid (T, H + 2G), one wave per (token, head): query heads, then key heads, then value heads. Element e < rot_dims
-// of a query / key head turns with its neighbour e ^ 1 by angle pos * base^(-(e / 2) * 2 / rot_dims).
+// grid (T, H + G + Gv), one wave per (token, head): query heads, then key heads, then the Gv value heads. Element
+// e < rot_dims of a query / key head turns with its neighbour e ^ 1 by angle pos * base^(-(e / 2) * 2 / rot_dims); with
+// `half` the pairs are (i, i + rot_dims / 2) instead and pair i turns by pos * base^(-i * 2 / rot_dims).
 constexpr int HEAD_E = 8;  // elements per lane: heads of up to 512 numbers
 template <bool Q16, bool C16>
 __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, const float* ki, const float* vi,
@@ -160,14 +161,15 @@ __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, c
                                                               int G, int dk, int dv, int rot, float neg_log_base,
                                                               int norm, float eps, void* qo, int ldqo, void* kc,
                                                               void* vc, const int* slots, const float* qw,
-                                                              const float* kw, float temp_coef, int temp_every) {
+                                                              const float* kw, float temp_coef, int temp_every,
+                                                              int half, int Gv) {
     const int t = blockIdx.x, u = blockIdx.y, lane = threadIdx.x;
     if (u >= H + G) {  // value head: plain copy into the pool
         const int sl = slots[t];
         if (sl < 0) return;
         const int g = u - H - G;
         const float* src = vi + (long)t * ldv + (long)g * dv;
-        const long dst = ((long)sl * G + g) * dv;
+        const long dst = ((long)sl * Gv + g) * dv;
         for (int e = lane; e < dv; e += 64) st_elem<C16>(vc, dst + e, src[e]);
         return;
     }
@@ -189,11 +191,15 @@ __global__ __launch_bounds__(64) void rope_norm_append_kernel(const float* qi, c
         if (e < dk) {
             v = src[e];
             if (e < rot) {
-                const float other = src[e ^ 1];
-                const float f = expf((float)(e >> 1) * (2.f / (float)rot) * neg_log_base);
+                const int n2 = rot >> 1;
+                const bool second = half ? e >= n2 : (e & 1);  // the pair's second member turns as v cos + u sin
+                const int mate = half ? (second ? e - n2 : e + n2) : (e ^ 1);
+                const int pi = half ? (second ? e - n2 : e) : (e >> 1);
+                const float other = src[mate];
+                const float f = expf((float)pi * (2.f / (float)rot) * neg_log_base);
                 float s, c;
                 sincosf(pos * f, &s, &c);
-                v = (e & 1) ? v * c + other * s : v * c - other * s;
+                v = second ? v * c + other * s : v * c - other * s;
             }
         }
         val[k] = v;
@@ -312,8 +318,10 @@ __global__ __launch_bounds__(NT) void scan_coefs_kernel(const float* a, int lda,
 
 // out = exp(log_sigmoid(x) * inv_tau) = sigmoid(x)^(1 / tau) with x = z + bias, or, with a projection proj [R, C],
 // x = sum_r z[t, r] proj[r, c] + bias[c] (the second half of a low-rank projection, summed in fp32 in a fixed order)
+// With rate_log (one per head of `per` channels): out = exp(-exp(rate_log[c / per]) * softplus(x)) instead.
 __global__ __launch_bounds__(NT) void channel_decay_kernel(const float* z, int ldz, const float* bias, float inv_tau,
-                                                           float* out, int C, const float* proj, int R) {
+                                                           float* out, int C, const float* proj, int R,
+                                                           const float* rate_log, int per) {
     extern __shared__ float zr[];  // the token's R inputs of the projection
     const int c = blockIdx.y * NT + threadIdx.x, t = blockIdx.x;
     if (proj) {
@@ -327,20 +335,52 @@ __global__ __launch_bounds__(NT) void channel_decay_kernel(const float* z, int l
     } else {
         x += z[(long)t * ldz + c];
     }
-    out[(long)t * C + c] = expf(-softplus_acc(-x) * inv_tau);
+    out[(long)t * C + c] = rate_log ? expf(-expf(rate_log[c / per]) * softplus_acc(x)) : expf(-softplus_acc(-x) * inv_tau);
 }
 
 // grid (T, C / group): one block per (token, group of columns). Groups of up to blockDim * GC numbers are read once
 // (straight-line clamped loads, all in flight together) and kept in registers with their gates; the launcher picks
 // the smallest GC that holds the group
+// sigm: the gate's activation is a sigmoid instead of a SiLU. proj [R, C]: the gate row holds R numbers and column
+// c's pre-activation is sum_r gate[t, r] proj[r, c], summed in fp32 in a fixed order (a low-rank gate's second half).
+MX_DEV float gate_act(float x, int sigm) { return sigm ? sigmoid_acc(x) : silu_acc(x); }
+MX_DEV float gate_pre(const float* gr, const float* proj, int R, int C, int c, const float* zr) {
+    if (!proj) return gr[c];
+    float x = 0.f;
+    for (int r = 0; r < R; ++r) x += zr[r] * proj[(long)r * C + c];
+    return x;
+}
 template <bool B16, int GC>
 __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
-                                        float eps, int group, int gate_first, float out_scale, void* out, int ldo) {
+                                        float eps, int group, int gate_first, float out_scale, void* out, int ldo,
+                                        int sigm, const float* proj, int R, int C) {
     __shared__ float red[16];
+    extern __shared__ float zr[];  // the token's R inputs of the gate projection
     const int t = blockIdx.x, c0 = blockIdx.y * group;
     const float* yr = y + (long)t * ldy + c0;
-    const float* gr = gate + (long)t * ldg + c0;
+    const float* gr = gate + (long)t * ldg + (proj ? 0 : c0);
     const int nt = blockDim.x;
+    if (proj) {  // the general form below, with the projected gate
+        for (int r = threadIdx.x; r < R; r += nt) zr[r] = gr[r];
+        __syncthreads();
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < group; e += nt) {
+            float v = yr[e];
+            if (gate_first) v *= gate_act(gate_pre(gr, proj, R, C, c0 + e, zr), sigm);
+            ss += v * v;
+        }
+        ss = block_sum_dyn(ss, red);
+        const float sc = out_scale / sqrtf(ss / (float)group + eps);
+        for (int e = threadIdx.x; e < group; e += nt) {
+            const float g = gate_act(gate_pre(gr, proj, R, C, c0 + e, zr), sigm);
+            float v = yr[e];
+            if (gate_first) v *= g;
+            v = v * sc * w[(c0 + e) % wlen];
+            if (!gate_first) v *= g;
+            st_elem<B16>(out, (long)t * ldo + c0 + e, v);
+        }
+        return;
+    }
     if (group <= nt * GC) {
         float z[GC], gs[GC];
         float ss = 0.f;
@@ -353,7 +393,7 @@ __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* ga
 #pragma unroll
         for (int k = 0; k < GC; ++k) {
             const int e = threadIdx.x + k * nt;
-            gs[k] = silu_acc(gs[k]);
+            gs[k] = gate_act(gs[k], sigm);
             z[k] = e < group ? (gate_first ? z[k] * gs[k] : z[k]) : 0.f;
             ss += z[k] * z[k];
         }
@@ -373,13 +413,13 @@ __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* ga
     float ss = 0.f;
     for (int e = threadIdx.x; e < group; e += nt) {
         float v = yr[e];
-        if (gate_first) v *= silu_acc(gr[e]);
+        if (gate_first) v *= gate_act(gr[e], sigm);
         ss += v * v;
     }
     ss = block_sum_dyn(ss, red);
     const float sc = out_scale / sqrtf(ss / (float)group + eps);
     for (int e = threadIdx.x; e < group; e += nt) {
-        const float g = silu_acc(gr[e]);
+        const float g = gate_act(gr[e], sigm);
         float v = yr[e];
         if (gate_first) v *= g;
         v = v * sc * w[(c0 + e) % wlen];
@@ -389,10 +429,14 @@ __global__ void gated_group_norm_kernel(const float* y, int ldy, const float* ga
 }
 
 // grid (T, ceil(F / NT))
+// act 0: silu(x) * y * factor; 1: gelu_tanh(x) * y * factor; 2 (no second operand): relu(factor * x)^2
+MX_DEV float gelu_tanh_acc(float x) {
+    return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
 template <bool B16>
 __global__ __launch_bounds__(NT) void glu_kernel(const float* a, int lda, const float* b, int ldb, const float* ba,
                                                  const float* bb, const float* scale, int lds, int group,
-                                                 int scale_sigmoid, void* out, int ldo, int F) {
+                                                 int scale_sigmoid, void* out, int ldo, int F, int act) {
     const int f = blockIdx.y * NT + threadIdx.x, t = blockIdx.x;
     if (f >= F) return;
     float fac = 1.f;
@@ -405,14 +449,20 @@ __global__ __launch_bounds__(NT) void glu_kernel(const float* a, int lda, const 
         }
     }
     const float x = a[(long)t * lda + f] + (ba ? ba[f] : 0.f);
+    if (act == 2) {
+        const float r = fmaxf(fac * x, 0.f);
+        st_elem<B16>(out, (long)t * ldo + f, r * r);
+        return;
+    }
     const float y = b[(long)t * ldb + f] + (bb ? bb[f] : 0.f);
-    st_elem<B16>(out, (long)t * ldo + f, silu_acc(x) * y * fac);
+    st_elem<B16>(out, (long)t * ldo + f, (act == 1 ? gelu_tanh_acc(x) : silu_acc(x)) * y * fac);
 }
 
 // one wave per token; lane l holds experts l, l + 64, ... (up to 16 each)
 constexpr int ROUTE_E = 16;
+// sigm: the chosen experts keep sigmoid(logit) * scale as their weights (no softmax, no renormalisation)
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int ld, const float* bias, int E, int top,
-                                                       float scale, float eps, float* weights) {
+                                                       float scale, float eps, float* weights, int sigm) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (long)t * ld;
     float v[ROUTE_E];
@@ -469,7 +519,10 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* logits, int 
 #pragma unroll
     for (int k = 0; k < ROUTE_E; ++k) {
         const int e = lane + k * 64;
-        if (e < E && v[k] < 0.f) wr[e] = mine[k] * norm;  // the taken ones (absent ones have e >= E)
+        if (e < E && v[k] < 0.f) {  // the taken ones (absent ones have e >= E)
+            // exp(z - m) orders the experts as their logits do, so the same `top` are taken in both modes
+            wr[e] = sigm ? scale * sigmoid_acc(z[e] + (bias ? bias[e] : 0.f)) : mine[k] * norm;
+        }
     }
 }
 
@@ -509,17 +562,19 @@ extern "C" int mxh_rope_norm_append(const float* qi, const float* ki, const floa
                                     const int* positions, int H, int G, int dk, int dv, int rot, float base, int norm,
                                     float eps, void* qo, int ldqo, int q16, void* kc, void* vc, int c16,
                                     const int* slots, const float* qw, const float* kw, float temp_coef,
-                                    int temp_every, int T, hipStream_t st) {
+                                    int temp_every, int half, int Gv, int T, hipStream_t st) {
     if (T <= 0) return 0;
     MXH_CHECK(qi && ki && vi && positions && qo && kc && vc && slots && temp_every >= 1);
-    // G == 0: queries only (keys and values of another layer are read)
-    MXH_CHECK(H > 0 && G >= 0 && dk > 0 && dv > 0 && dk <= 64 * HEAD_E && rot >= 0 && rot <= dk && rot % 2 == 0);
-    MXH_CHECK(ldq >= H * dk && ldk >= G * dk && ldv >= G * dv && ldqo >= H * dk && base > 0.f);
-    const dim3 grid(T, H + 2 * G);
+    // G == 0: queries only (keys and values of another layer are read). Gv value heads (the pool's row is Gv * dv)
+    MXH_CHECK(H > 0 && G >= 0 && Gv >= 0 && (G > 0) == (Gv > 0) && dk > 0 && dv > 0 && dk <= 64 * HEAD_E && rot >= 0 &&
+              rot <= dk && rot % 2 == 0);
+    MXH_CHECK(ldq >= H * dk && ldk >= G * dk && ldv >= Gv * dv && ldqo >= H * dk && base > 0.f && H + G + Gv <= 65535);
+    const dim3 grid(T, H + G + Gv);
     const float nlb = -logf(base);
 #define GO(Q, C)                                                                                                   \
     rope_norm_append_kernel<Q, C><<<grid, 64, 0, st>>>(qi, ki, vi, ldq, ldk, ldv, positions, H, G, dk, dv, rot, nlb, \
-                                                       norm, eps, qo, ldqo, kc, vc, slots, qw, kw, temp_coef, temp_every)
+                                                       norm, eps, qo, ldqo, kc, vc, slots, qw, kw, temp_coef, temp_every, \
+                                                       half, Gv)
     if (q16 && c16) GO(true, true);
     else if (q16) GO(true, false);
     else if (c16) GO(false, true);
@@ -562,24 +617,26 @@ extern "C" int mxh_scan_coefs(const float* a, int lda, const float* b, int ldb, 
 }
 
 extern "C" int mxh_channel_decay(const float* z, int ldz, const float* bias, float inv_tau, float* out, int T, int C,
-                                 const float* proj, int R, hipStream_t st) {
+                                 const float* proj, int R, const float* rate_log, int per, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(z && out && C > 0 && inv_tau > 0.f && C <= 65535 * NT);
+    MXH_CHECK(z && out && C > 0 && inv_tau > 0.f && C <= 65535 * NT && (!rate_log || (per > 0 && C % per == 0)));
     MXH_CHECK(proj ? (R > 0 && R <= 8192 && ldz >= R) : ldz >= C);
     channel_decay_kernel<<<dim3(T, (C + NT - 1) / NT), NT, proj ? R * sizeof(float) : 0, st>>>(z, ldz, bias, inv_tau, out,
-                                                                                            C, proj, R);
+                                                                                            C, proj, R, rate_log, per);
     return (int)hipGetLastError();
 }
 
 extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, int ldg, const float* w, int wlen,
                                     float eps, int group, int gate_first, float out_scale, void* out, int ldo,
-                                    int o16, int T, int C, hipStream_t st) {
+                                    int o16, int T, int C, int sigm, const float* proj, int R, hipStream_t st) {
     if (T <= 0) return 0;
     MXH_CHECK(y && gate && w && out && C > 0 && group > 0 && C % group == 0 && wlen > 0 && C % wlen == 0);
-    MXH_CHECK(ldy >= C && ldg >= C && ldo >= C);
+    MXH_CHECK(ldy >= C && ldo >= C && (proj ? (R > 0 && R <= 8192 && ldg >= R) : ldg >= C) && C / group <= 65535);
     const dim3 grid(T, C / group);
-#define GO(B, G_, nt_) \
-    gated_group_norm_kernel<B, G_><<<grid, nt_, 0, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, out, ldo)
+    const size_t dyn = proj ? R * sizeof(float) : 0;
+#define GO(B, G_, nt_)                                                                                              \
+    gated_group_norm_kernel<B, G_><<<grid, nt_, dyn, st>>>(y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, \
+                                                           out, ldo, sigm, proj, R, C)
 #define PICK(B)                              \
     do {                                     \
         if (group <= 256) GO(B, 4, 64);      \
@@ -596,20 +653,23 @@ extern "C" int mxh_gated_group_norm(const float* y, int ldy, const float* gate, 
 
 extern "C" int mxh_glu(const float* a, int lda, const float* b, int ldb, const float* ba, const float* bb,
                        const float* scale, int lds, int group, int scale_sigmoid, void* out, int ldo, int o16, int T,
-                       int F, hipStream_t st) {
+                       int F, int act, hipStream_t st) {
     if (T <= 0 || F <= 0) return 0;
-    MXH_CHECK(a && b && out && lda >= F && ldb >= F && ldo >= F && group > 0 && F <= 65535 * NT);
+    MXH_CHECK(a && out && lda >= F && ldo >= F && group > 0 && F <= 65535 * NT && act >= 0 && act <= 2);
+    MXH_CHECK(act == 2 ? !b : (b && ldb >= F));  // the squared ReLU has one operand
     MXH_CHECK(!scale || (F % group == 0 && lds >= F / group));
     const dim3 grid(T, (F + NT - 1) / NT);
-    if (o16) glu_kernel<true><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F);
-    else glu_kernel<false><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F);
+    if (o16)
+        glu_kernel<true><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F, act);
+    else
+        glu_kernel<false><<<grid, NT, 0, st>>>(a, lda, b, ldb, ba, bb, scale, lds, group, scale_sigmoid, out, ldo, F, act);
     return (int)hipGetLastError();
 }
 
 extern "C" int mxh_moe_route(const float* logits, int ld, const float* bias, int T, int E, int top, float scale,
-                             float eps, float* weights, hipStream_t st) {
+                             float eps, float* weights, int sigm, hipStream_t st) {
     if (T <= 0) return 0;
     MXH_CHECK(logits && weights && E > 0 && E <= 64 * ROUTE_E && top > 0 && top <= E && ld >= E);
-    moe_route_kernel<<<T, 64, 0, st>>>(logits, ld, bias, E, top, scale, eps, weights);
+    moe_route_kernel<<<T, 64, 0, st>>>(logits, ld, bias, E, top, scale, eps, weights, sigm);
     return (int)hipGetLastError();
 }

@@ -12,7 +12,10 @@
 // sequence's slot unless the chunk starts at position 0, and written back after the chunk's last row: a decode row is
 // a chunk of one, a prompt chunk walks its rows inside one launch.
 // CHD (gated linear attention): the decay is one number per head and state row, a_t[n], staged beside k_t and q_t:
-// S[n][p] <- a_t[n] S[n][p] + k_t[n] u[p]. A missing write strength means 1; q_t is multiplied by q_scale when staged.
+// S[n][p] <- a_t[n] S[n][p] + k_t[n] u[p]; with DELTA as well, the delta rule's read follows that per-row decay. A
+// missing write strength means 1, one given as pre-activations (coef_sigmoid, row stride ldc) passes a sigmoid when
+// staged; q_t is multiplied by q_scale when staged. A decay row stride of 0 (ldd) is one constant per head for every
+// token (retention).
 #include "../mx_common.h"
 
 namespace {
@@ -36,7 +39,8 @@ MX_DEV float lanes_sum(float v) {
 // grid (column blocks, H, sequences); block = 256 threads = 256 / LPC columns
 template <int NPL, int LPC, bool DELTA, bool CHD>
 __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk, const float* q, int ldq,
-                                                         const float* v, int ldv, const float* decay, const float* coef,
+                                                         const float* v, int ldv, const float* decay, int ldd,
+                                                         const float* coef, int ldc, int coef_sigmoid,
                                                          const float* skip, float* state, const int* seq_state,
                                                          const int* positions, int n_dec, const int* pf_cu, float* out,
                                                          int ldo, int H, int G, int N, int P, float q_scale) {
@@ -130,8 +134,12 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
         }
         if (threadIdx.x < 2 * TB) {
             const long row = min(r0 + (int)threadIdx.x / 2, last);
-            if (threadIdx.x & 1) st_ac = coef ? coef[row * H + h] : 1.f;
-            else st_ac = CHD ? 1.f : decay[row * H + h];
+            if (threadIdx.x & 1) {
+                st_ac = coef ? coef[row * ldc + h] : 1.f;
+                if (coef && coef_sigmoid) st_ac = 1.f / (1.f + expf(-st_ac));
+            } else {
+                st_ac = CHD ? 1.f : decay[row * ldd + h];
+            }
         }
     };
     auto publish = [&](int b) {
@@ -159,10 +167,11 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
             float u;
             if constexpr (DELTA) {
                 float d0 = 0.f, d1 = 0.f;  // two chains instead of one of NPL dependent adds
+                const float* ab = &kq[b][tt][NW - 1][part * NPL];  // (the channel decays; q's row when there are none)
 #pragma unroll
                 for (int j = 0; j < NPL; j += 2) {
-                    S[j] *= a;
-                    S[j + 1] *= a;
+                    S[j] *= CHD ? ab[j] : a;
+                    S[j + 1] *= CHD ? ab[j + 1] : a;
                     d0 += S[j] * kb[j];
                     d1 += S[j + 1] * kb[j + 1];
                 }
@@ -211,14 +220,15 @@ __global__ __launch_bounds__(256) void state_scan_kernel(const float* k, int ldk
     if (!(cond)) return (int)hipErrorInvalidValue
 
 extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, const float* v, int ldv,
-                              const float* decay, const float* coef, const float* skip, float* state,
-                              const int* seq_state, const int* positions, int n_dec, const int* pf_cu, int n_pf,
-                              float* out, int ldo, int H, int G, int N, int P, int delta, int channel, float q_scale,
-                              hipStream_t st) {
+                              const float* decay, int decay_rows, const float* coef, int ldc, int coef_sigmoid,
+                              const float* skip, float* state, const int* seq_state, const int* positions, int n_dec,
+                              const int* pf_cu, int n_pf, float* out, int ldo, int H, int G, int N, int P, int delta,
+                              int channel, float q_scale, hipStream_t st) {
     const int n_seqs = n_dec + n_pf;
     if (n_seqs <= 0) return 0;
     MXH_CHECK(k && q && v && decay && state && seq_state && positions && out && (n_pf == 0 || pf_cu));
-    MXH_CHECK(!(delta && channel));
+    MXH_CHECK((decay_rows || !channel) && (!coef || ldc >= H));  // decay_rows 0: one constant per head, [H]
+    const int ldd = decay_rows ? H : 0;
     MXH_CHECK(H > 0 && G > 0 && H % G == 0 && N > 0 && N <= 256 && P > 0 && H <= 65535 && n_seqs <= 65535);
     MXH_CHECK(ldk >= G * N && ldq >= G * N && ldv >= H * P && ldo >= H * P);
     const int lpc = N <= 32 ? 4 : 16;
@@ -226,12 +236,13 @@ extern "C" int mxh_state_scan(const float* k, int ldk, const float* q, int ldq, 
     const int cols = threads / lpc;
     const dim3 grid((P + cols - 1) / cols, H, n_seqs);
 #define GO2(NPL, LPC, D_, C_)                                                                                      \
-    state_scan_kernel<NPL, LPC, D_, C_><<<grid, threads, 0, st>>>(k, ldk, q, ldq, v, ldv, decay, coef, skip, state,    \
-                                                                  seq_state, positions, n_dec, pf_cu, out, ldo, H, G, \
-                                                                  N, P, q_scale)
+    state_scan_kernel<NPL, LPC, D_, C_><<<grid, threads, 0, st>>>(k, ldk, q, ldq, v, ldv, decay, ldd, coef, ldc,      \
+                                                                  coef_sigmoid, skip, state, seq_state, positions,    \
+                                                                  n_dec, pf_cu, out, ldo, H, G, N, P, q_scale)
 #define GO(NPL, LPC)                              \
     do {                                          \
-        if (delta) GO2(NPL, LPC, true, false);    \
+        if (delta && channel) GO2(NPL, LPC, true, true); \
+        else if (delta) GO2(NPL, LPC, true, false);   \
         else if (channel) GO2(NPL, LPC, false, true); \
         else GO2(NPL, LPC, false, false);         \
     } while (0)

@@ -150,26 +150,28 @@ HYBRID_SIGS = {
     "mxh_norm_add": [P, I, P, F, F, P, I, P, I, I, I, P],
     # q, k, v, ldq, ldk, ldv, positions, H, G, dk, dv, rot_dims, base, norm, eps, q_out, ldqo, q16, kc, vc, c16, slots,
     # q_weight, k_weight, temp_coef, temp_every, T, stream
-    "mxh_rope_norm_append": [P, P, P, I, I, I, P, I, I, I, I, I, F, I, F, P, I, I, P, P, I, P, P, P, F, I, I, P],
+    # ..., temp_every, half, value heads, T, stream
+    "mxh_rope_norm_append": [P, P, P, I, I, I, P, I, I, I, I, I, F, I, F, P, I, I, P, P, I, P, P, P, F, I, I, I, I, P],
     # q, ldq, q16, kc, vc, bs, bt, bt_stride, cu_q, ctx, n_seqs, n_rows, row_base, out, ldo, o16, H, G, dk, dv, scale,
     # chunk, window, sink, out_scale, row_off, parts, part_len, part_ml, part_o, sink_v, bias, bias_rows, gate, ldg,
     # stream
+    # (value heads before the stream)
     "mxh_attention": [P, I, I, P, P, I, P, I, P, P, I, I, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, I, P, P, P, P, I,
-                      P, I, P],
+                      P, I, I, P],
     # q, ldq, kc, vc, bs, table, p0, n, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale, sink_v,
     # bias, bias_rows, gate, ldg, stream
-    "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P, P, I, P, I, P],
+    "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P, P, I, P, I, I, P],
     "mxh_attention_mfma_ok": [I, I],
     # q, ldq, kc, vc, bs, bt, bt_stride, ctx, n_seqs, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale,
     # parts, part_len, part_ml, part_o, sink_v, bias, bias_rows, gate, ldg, stream
     "mxh_attention_decode_mfma": [P, I, P, P, I, P, I, P, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, P, P, P, P, I, P,
-                                  I, P],
+                                  I, I, P],
     # kc, vc, is16, bs, table, lo, n, G, dk, dv, kh, vh, stream
-    "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, P],
+    "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, I, P],
     # src, s16, s_stride_i, s_stride_h, dst, d16, d_stride_i, d_stride_h, n, H, d, scale, gate, ldg, stream
     "mxh_head_transpose": [P, I, L, L, P, I, L, L, I, I, I, F, P, I, P],
     # scores, weights, w16, rows, n, nk, p0, key0, scale, chunk, window, sink, sink_v, bias, bias_rows, H, stream
-    "mxh_masked_softmax": [P, P, I, L, I, I, I, I, F, I, I, I, P, P, I, I, P],
+    "mxh_masked_softmax": [P, P, I, L, I, I, I, I, F, I, I, I, P, P, I, I, I, P],
     # x, ldx, w, bias, taps, silu, tails, state, positions, n_dec, pf_cu, n_pf, out, ldo, T, C, stream
     "mxh_causal_conv": [P, I, P, P, I, I, P, P, P, I, P, I, P, I, I, I, P],
     # x, ldx, heads, dim, eps, scale, split, scale2, T, stream
@@ -177,16 +179,25 @@ HYBRID_SIGS = {
     # a, lda, b, ldb, A_log, dt_bias, decay, coef, T, H, stream
     "mxh_scan_coefs": [P, I, P, I, P, P, P, P, I, I, P],
     # z, ldz, bias, 1 / tau, out, T, C, proj, R, stream
-    "mxh_channel_decay": [P, I, P, F, P, I, I, P, I, P],
+    "mxh_channel_decay": [P, I, P, F, P, I, I, P, I, P, I, P],
     # k, ldk, q, ldq, v, ldv, decay, coef, skip, state, seq_state, positions, n_dec, pf_cu, n_pf, out, ldo, H, G, N, P,
     # delta, channel, q_scale, stream
-    "mxh_state_scan": [P, I, P, I, P, I, P, P, P, P, P, P, I, P, I, P, I, I, I, I, I, I, I, F, P],
-    # y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, out, ldo, o16, T, C, stream
-    "mxh_gated_group_norm": [P, I, P, I, P, I, F, I, I, F, P, I, I, I, I, P],
-    # a, lda, b, ldb, bias_a, bias_b, scale, lds, group, scale_sigmoid, out, ldo, o16, T, F, stream
-    "mxh_glu": [P, I, P, I, P, P, P, I, I, I, P, I, I, I, I, P],
-    # logits, ld, bias, T, E, top, scale, eps, weights, stream
-    "mxh_moe_route": [P, I, P, I, I, I, F, F, P, P],
+    "mxh_state_scan": [P, I, P, I, P, I, P, I, P, I, I, P, P, P, P, I, P, I, P, I, I, I, I, I, I, I, F, P],
+    # y, ldy, gate, ldg, w, wlen, eps, group, gate_first, out_scale, out, ldo, o16, T, C, sigmoid gate, proj, R, stream
+    "mxh_gated_group_norm": [P, I, P, I, P, I, F, I, I, F, P, I, I, I, I, I, P, I, P],
+    # a, lda, b, ldb, bias_a, bias_b, scale, lds, group, scale_sigmoid, out, ldo, o16, T, F, act, stream
+    "mxh_glu": [P, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, P],
+    # logits, ld, bias, T, E, top, scale, eps, weights, sigmoid scores, stream
+    "mxh_moe_route": [P, I, P, I, I, I, F, F, P, I, P],
+    # table, pair, is16, V, tokens, seq_state, positions, n_dec, pf_cu, n_pf, last, scale, mul_prev, mul_cur, buckets,
+    # out, copies, T, C, stream
+    "mxh_embed_pair": [P, P, I, I, P, P, P, I, P, I, P, F, I, I, I, P, I, I, I, P],
+    # xs, y, ldy, mix, out_w, in_w, norm_w, offset, eps, h32, ld32, h16, ld16, total, ldt, T, S, C, stream
+    "mxh_hyper_step": [P, P, I, P, P, P, P, F, F, P, I, P, I, P, I, I, I, I, P],
+    # x, ldx, positions, heads, dim, rot_dims, base, half, scale, split, scale2, T, stream
+    "mxh_rope_rows": [P, I, P, I, I, I, F, I, F, I, F, I, P],
+    # a, lda, b, ldb, lam, eps, group, out_scale, out, ldo, o16, T, C, stream
+    "mxh_diff_group_norm": [P, I, P, I, F, F, I, F, P, I, I, I, I, P],
 }
 
 HIP_ERRORS = {1: "hipErrorInvalidValue", 2: "hipErrorOutOfMemory", 98: "hipErrorInvalidDeviceFunction",

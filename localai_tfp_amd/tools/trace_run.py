@@ -28,7 +28,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True)
     ap.add_argument("--max-seqs", type=int, default=4)
     ap.add_argument("--block-size", type=int, default=16)
-    ap.add_argument("--device", default=None, help="cuda (default when a GPU is present) or cpu")
+    ap.add_argument("--device", default="cuda", help="cuda (default), or cpu for the fp32 plumbing path without kernels")
     a = ap.parse_args(argv)
 
     import numpy as np
@@ -36,8 +36,11 @@ def main(argv=None) -> int:
     from ..engine.engine import EngineConfig, LLMEngine
     from ..models.loader import load_llm
 
-    dev = a.device or ("cuda" if torch.cuda.is_available() else "cpu")
+    dev = a.device
     if dev.startswith("cuda"):  # the model's kernel library is built at its first launch if the tree has none
+        if not torch.cuda.is_available():  # never a silent CPU run: the kernels are what a replay is about
+            print("trace_run: no GPU is visible (pass --device cpu for the plumbing path)", file=sys.stderr)
+            return 2
         torch.backends.cuda.matmul.allow_tf32 = False
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[a.dtype]
     model, tok, _cfg, _ = load_llm(a.model, torch.device(dev), overrides={"dtype": dtype})
