@@ -96,13 +96,13 @@ def parse():
                     help="comma list of sampling phases measured back to back on the same server: reference = "
                          "the reference's defaults (temperature 0.9, top_k 40, top_p 0.95; backend_config.go "
                          "SetDefaults) on the GPU sampler; greedy = argmax. The first phase is the headline")
-    ap.add_argument("--arch-bench", default="", choices=["", "vosotar", "vugotar", "girulorn"],
+    ap.add_argument("--arch-bench", default="", choices=["", "vosotar", "vugotar", "girulorn", "keronex"],
                     help="instead of the headline serving benchmark: prefill and decode throughput of this model "
                          "family beside the Llama graph at equal layer sizes (random bf16 / f16 weights, one GPU)")
     ap.add_argument("--arch-sizes", default="1b,7b", help="--arch-bench: comma list of layer sizes (1b, 7b)")
     ap.add_argument("--arch-layers", type=int, default=4, help="--arch-bench: layers per model")
     ap.add_argument("--arch-models", default="", help="--arch-bench: comma list to restrict the models (vosotar, vugotar, girulorn, "
-                         "vugotar-moe, llama-f16)")
+                         "keronex, vugotar-moe, llama-f16)")
     ap.add_argument("--arch-batches", default="1,32", help="--arch-bench: decode batch sizes")
     ap.add_argument("--arch-chunk", type=int, default=2048, help="--arch-bench vugotar: attention chunk size")
     return ap.parse_args()
@@ -252,6 +252,30 @@ def run_arch_bench(args) -> int:
                                 g_heads=s["heads"] // 2, g_dim=128, g_vdim=128, tau=12.0, rank=32,
                                 name=f"girulorn-{sz}", **moe)
             yield "girulorn", lambda: GI.GirulornModel.load(gc, GI.synthetic_source(gc, 1), dev, torch.bfloat16)
+            pat = tuple("mamba2" if i % 4 == 3 else "parallel" for i in range(nl))
+            uc = VU.make_config(hidden=s["hidden"], vocab=V, pattern=pat, mlps=("moe",), heads=s["heads"],
+                                kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, chunk=args.arch_chunk,
+                                d_heads=s["heads"] // 2, d_kv_heads=max(1, s["heads"] // 4), d_dim=128, d_vdim=128,
+                                d_conv=4, m_heads=2 * s["hidden"] // 64, m_vdim=64, m_state=128, m_groups=1,
+                                m_norm_groups=1, m_conv=4, name=f"vugotar-{sz}", **moe)
+            yield "vugotar-moe", lambda: VU.VugotarModel.load(uc, VU.synthetic_source(uc, 1), dev, torch.bfloat16)
+        elif args.arch_bench == "keronex":
+            # one differential-attention layer, two delta-rule layers with per-channel decays and a retention layer in
+            # turn, on four residual streams; attention heads as the Llama graph's (GQA 4:1) with two maps of 64 numbers
+            # each over values of 128, half as many recurrent heads with 128 x 128 states; 8 experts of a quarter of the
+            # feed-forward width, two chosen, and a shared expert of half of it. The closest model of the framework,
+            # Vugotar (attention beside a delta rule with a short convolution, a state-space layer every fourth), runs
+            # beside it with expert feed-forwards of the same widths.
+            from localai_tfp_amd.models import keronex as KE
+            from localai_tfp_amd.models import vugotar as VU
+            kinds = ("attention", "channel_delta", "channel_delta", "retention")
+            moe = dict(experts=8, top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 2)
+            kc = KE.make_config(hidden=s["hidden"], vocab=V, pattern=tuple(kinds[i % 4] for i in range(nl)),
+                                heads=s["heads"], kv_heads=max(1, s["heads"] // 4), dim=64, vdim=128, rot_dims=64,
+                                r_heads=s["heads"] // 2, r_dim=128, r_vdim=128, d_heads=s["heads"] // 2,
+                                d_kv_heads=s["heads"] // 2, d_dim=128, d_vdim=128, conv=4, rank_a=32, rank_g=32,
+                                mlps=("moe",), streams=4, bigram=(65521, 1009, 31), name=f"keronex-{sz}", **moe)
+            yield "keronex", lambda: KE.KeronexModel.load(kc, KE.synthetic_source(kc, 1), dev, torch.bfloat16)
             pat = tuple("mamba2" if i % 4 == 3 else "parallel" for i in range(nl))
             uc = VU.make_config(hidden=s["hidden"], vocab=V, pattern=pat, mlps=("moe",), heads=s["heads"],
                                 kv_heads=max(1, s["heads"] // 4), dim=128, vdim=128, chunk=args.arch_chunk,

@@ -323,7 +323,9 @@ MX_DEV bf16x8 v_fragment(const char* v_lds, int r0, int nt, int col) {
 // fragments coming out of LDS through the transposing read.
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (g = lane / 16, col = lane % 16): A holds row col, k = 8g .. 8g + 7;
 // B holds column col, k = 8g .. 8g + 7; the result holds rows 4g .. 4g + 3 of column col.
-template <int DK, int DV, bool O16>
+// P2: every softmax weight enters the value product as two bf16 numbers (its rounding, and the rounding of what that
+// lost) in two products that share the value fragment, so the weights count to 16 bits of mantissa.
+template <int DK, int DV, bool O16, bool P2>
 __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __restrict__ q, int ldq,
                                                               const bf16_t* __restrict__ kc,
                                                               const bf16_t* __restrict__ vc, int bs,
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
     constexpr float LOG2E_ = 1.4426950408889634f;
     __shared__ __attribute__((aligned(16))) char k_lds[KT * KSTR];
     __shared__ __attribute__((aligned(16))) char v_lds[KT * VSTR];
-    __shared__ __attribute__((aligned(16))) char p_lds[4 * 16 * PSTR];
+    __shared__ __attribute__((aligned(16))) char p_lds[(P2 ? 2 : 1) * 4 * 16 * PSTR];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = lane >> 4, col = lane & 15;
     const int RT = 4 / GW;
@@ -373,6 +375,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
         lo_row[i] = chunk > 0 ? (qpos / chunk) * chunk : window > 0 ? max(0, qpos - window + 1) : 0;
     }
     char* pw = p_lds + wave * 16 * PSTR;
+    char* pw2 = pw + (P2 ? 4 * 16 * PSTR : 0);  // the weights' second halves
 
     constexpr int KCH = KT * DK / 8 / 256, VCH = KT * DV / 8 / 256;  // 16-byte pieces per thread
     u32x4 kr[KCH], vr[VCH];
@@ -455,18 +458,25 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i]);
+            for (int i = 0; i < 4; ++i) {
+                const bf16_t hi = f32_to_bf16(sacc[t][i]);
+                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = hi;
+                if constexpr (P2)
+                    *(bf16_t*)(pw2 + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i] - bf16_to_f32(hi));
+            }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
         __builtin_amdgcn_wave_barrier();
         // ---- O += P V ----
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (32 * ks + 8 * g) * 2);
+            const bf16x8 pb = *(const bf16x8*)(pw2 + col * PSTR + (32 * ks + 8 * g) * 2);
 #pragma unroll
-            for (int nt = 0; nt < DV / 16; ++nt)
-                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col),
-                                                                   oacc[nt], 0, 0, 0);
+            for (int nt = 0; nt < DV / 16; ++nt) {
+                const auto vf = v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col);
+                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vf, oacc[nt], 0, 0, 0);
+                if constexpr (P2) oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb, vf, oacc[nt], 0, 0, 0);
+            }
         }
         __syncthreads();
     }
@@ -492,7 +502,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const bf16_t* __re
 // wave itself, the next tile requested ahead). With one
 // partition it writes the result, otherwise (max, sum, unnormalised output) for attn_merge_kernel; the running maximum
 // is kept in base 2 and handed over in base e.
-template <int DK, int DV, bool O16>
+template <int DK, int DV, bool O16, bool P2>
 __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __restrict__ q, int ldq,
                                                               const bf16_t* __restrict__ kc,
                                                               const bf16_t* __restrict__ vc, int bs,
@@ -506,7 +516,8 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
     constexpr int VSTR = (DV + 8) * 2, PSTR = (KT + 8) * 2;
     constexpr float LOG2E_ = 1.4426950408889634f, LN2_ = 0.6931471805599453f;
     __shared__ __attribute__((aligned(16))) char v_lds[KT * VSTR];
-    __shared__ __attribute__((aligned(16))) char pw[16 * PSTR];
+    __shared__ __attribute__((aligned(16))) char pw[(P2 ? 2 : 1) * 16 * PSTR];
+    char* pw2 = pw + (P2 ? 16 * PSTR : 0);  // the weights' second halves (P2 as in attn_chunk_mfma_kernel)
     const int lane = threadIdx.x, g = lane >> 4, col = lane & 15;
     const int s = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
     const int rep = H / G;
@@ -631,16 +642,23 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(const bf16_t* __re
 #pragma unroll
         for (int t = 0; t < KT / 16; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i]);
+            for (int i = 0; i < 4; ++i) {
+                const bf16_t hi = f32_to_bf16(sacc[t][i]);
+                *(bf16_t*)(pw + (4 * g + i) * PSTR + (16 * t + col) * 2) = hi;
+                if constexpr (P2)
+                    *(bf16_t*)(pw2 + (4 * g + i) * PSTR + (16 * t + col) * 2) = f32_to_bf16(sacc[t][i] - bf16_to_f32(hi));
+            }
         __syncthreads();
 #pragma unroll
         for (int ks = 0; ks < KT / 32; ++ks) {
             const bf16x8 pa = *(const bf16x8*)(pw + col * PSTR + (32 * ks + 8 * g) * 2);
+            const bf16x8 pb = *(const bf16x8*)(pw2 + col * PSTR + (32 * ks + 8 * g) * 2);
 #pragma unroll
-            for (int nt = 0; nt < DV / 16; ++nt)
-                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col),
-                                                                   oacc[nt], 0, 0, 0);
+            for (int nt = 0; nt < DV / 16; ++nt) {
+                const auto vf = v_fragment<VSTR>(v_lds, 32 * ks + 8 * g, nt, col);
+                oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vf, oacc[nt], 0, 0, 0);
+                if constexpr (P2) oacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pb, vf, oacc[nt], 0, 0, 0);
+            }
         }
     }
 #pragma unroll
@@ -880,7 +898,8 @@ extern "C" int mxh_attention_mfma_ok(int dk, int dv) { return (dk == 64 || dk ==
 extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const void* vc, int bs, const int* table,
                                   int p0, int n, void* out, int ldo, int o16, int H, int G, int dk, int dv,
                                   float scale, int chunk, int window, int sink, float out_scale, const float* sink_v,
-                                  const float* bias, int nb, const float* gate, int ldg, int gv, hipStream_t st) {
+                                  const float* bias, int nb, const float* gate, int ldg, int gv, int p2,
+                                  hipStream_t st) {
     if (n <= 0) return 0;
     MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink) && gv > 0 && G % gv == 0);
     const AttnExtra ex = {sink_v, bias, nb, gate, ldg, gv};
@@ -891,22 +910,23 @@ extern "C" int mxh_attention_mfma(const void* q, int ldq, const void* kc, const 
     const int RT = 4 / GW;
     MXH_CHECK(H / GW <= 65535);
     const dim3 grid((n + RT * 16 - 1) / (RT * 16), H / GW);
-#define GO(K_, V_)                                                                                                    \
-    do {                                                                                                              \
-        if (o16)                                                                                                      \
-            attn_chunk_mfma_kernel<K_, V_, true><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,       \
-                                                                       (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
-                                                                       H, G, GW, scale, chunk, window, sink, out_scale, ex); \
-        else                                                                                                          \
-            attn_chunk_mfma_kernel<K_, V_, false><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,      \
-                                                                        (const bf16_t*)vc, bs, table, p0, n, out, ldo, \
-                                                                        H, G, GW, scale, chunk, window, sink, out_scale, ex); \
+#define GO3(K_, V_, O_, P_)                                                                                       \
+    attn_chunk_mfma_kernel<K_, V_, O_, P_><<<grid, 256, 0, st>>>((const bf16_t*)q, ldq, (const bf16_t*)kc,             \
+                                                                 (const bf16_t*)vc, bs, table, p0, n, out, ldo, H, G, \
+                                                                 GW, scale, chunk, window, sink, out_scale, ex)
+#define GO(K_, V_)                                 \
+    do {                                           \
+        if (o16 && p2) GO3(K_, V_, true, true);    \
+        else if (o16) GO3(K_, V_, true, false);    \
+        else if (p2) GO3(K_, V_, false, true);     \
+        else GO3(K_, V_, false, false);            \
     } while (0)
     if (dk == 64 && dv == 64) GO(64, 64);
     else if (dk == 64 && dv == 128) GO(64, 128);
     else if (dk == 128 && dv == 64) GO(128, 64);
     else GO(128, 128);
 #undef GO
+#undef GO3
     return (int)hipGetLastError();
 }
 
@@ -917,7 +937,7 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
                                          int G, int dk, int dv, float scale, int chunk, int window, int sink,
                                          float out_scale, int parts, int part_len, float* part_ml, float* part_o,
                                          const float* sink_v, const float* bias, int nb, const float* gate, int ldg,
-                                         int gv, hipStream_t st) {
+                                         int gv, int p2, hipStream_t st) {
     if (n_seqs <= 0) return 0;
     MXH_CHECK((!bias || nb > 0) && (!gate || ldg >= H) && (!sink_v || sink) && gv > 0 && G % gv == 0);
     const AttnExtra ex = {sink_v, bias, nb, gate, ldg, gv};
@@ -925,22 +945,23 @@ extern "C" int mxh_attention_decode_mfma(const void* q, int ldq, const void* kc,
     MXH_CHECK(H / G <= 16 && G <= 65535 && mxh_attention_mfma_ok(dk, dv) && ldq >= H * dk && ldq % 8 == 0 && ldo >= H * dv);
     MXH_CHECK(parts >= 1 && parts <= 64 && (parts == 1 || (part_len > 0 && part_ml && part_o)) && chunk >= 0 && window >= 0);
     const dim3 grid(n_seqs, G, parts);
-#define GO(K_, V_)                                                                                                       \
-    do {                                                                                                                 \
-        if (o16)                                                                                                         \
-            attn_decode_mfma_kernel<K_, V_, true><<<grid, 64, 0, st>>>(                                                  \
-                (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
-                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o, ex);                                       \
-        else                                                                                                             \
-            attn_decode_mfma_kernel<K_, V_, false><<<grid, 64, 0, st>>>(                                                 \
-                (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, \
-                chunk, window, sink, out_scale, parts, part_len, part_ml, part_o, ex);                                       \
+#define GO3(K_, V_, O_, P_)                                                                                             \
+    attn_decode_mfma_kernel<K_, V_, O_, P_><<<grid, 64, 0, st>>>(                                                           \
+        (const bf16_t*)q, ldq, (const bf16_t*)kc, (const bf16_t*)vc, bs, bt, bt_stride, ctx, out, ldo, H, G, scale, chunk, \
+        window, sink, out_scale, parts, part_len, part_ml, part_o, ex)
+#define GO(K_, V_)                                 \
+    do {                                           \
+        if (o16 && p2) GO3(K_, V_, true, true);    \
+        else if (o16) GO3(K_, V_, true, false);    \
+        else if (p2) GO3(K_, V_, false, true);     \
+        else GO3(K_, V_, false, false);            \
     } while (0)
     if (dk == 64 && dv == 64) GO(64, 64);
     else if (dk == 64 && dv == 128) GO(64, 128);
     else if (dk == 128 && dv == 64) GO(128, 64);
     else GO(128, 128);
 #undef GO
+#undef GO3
     if (parts > 1) {
         const dim3 g2(n_seqs, H);
         if (o16) attn_merge_kernel<true><<<g2, 64, 0, st>>>(part_ml, part_o, parts, H, dv, sink, out_scale, 0, out, ldo, ex);

@@ -160,12 +160,13 @@ HYBRID_SIGS = {
                       P, I, I, P],
     # q, ldq, kc, vc, bs, table, p0, n, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale, sink_v,
     # bias, bias_rows, gate, ldg, stream
-    "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P, P, I, P, I, I, P],
+    # (value heads and the two-part weights flag before the stream)
+    "mxh_attention_mfma": [P, I, P, P, I, P, I, I, P, I, I, I, I, I, I, F, I, I, I, F, P, P, I, P, I, I, I, P],
     "mxh_attention_mfma_ok": [I, I],
     # q, ldq, kc, vc, bs, bt, bt_stride, ctx, n_seqs, out, ldo, o16, H, G, dk, dv, scale, chunk, window, sink, out_scale,
     # parts, part_len, part_ml, part_o, sink_v, bias, bias_rows, gate, ldg, stream
     "mxh_attention_decode_mfma": [P, I, P, P, I, P, I, P, I, P, I, I, I, I, I, I, F, I, I, I, F, I, I, P, P, P, P, I, P,
-                                  I, I, P],
+                                  I, I, I, P],
     # kc, vc, is16, bs, table, lo, n, G, dk, dv, kh, vh, stream
     "mxh_kv_gather": [P, P, I, I, P, I, I, I, I, I, P, P, I, P],
     # src, s16, s_stride_i, s_stride_h, dst, d16, d_stride_i, d_stride_h, n, H, d, scale, gate, ldg, stream

@@ -401,10 +401,8 @@ class KeronexModel:
             elif L.type == "retention":
                 spec.append({"state": (m.heads, m.vdim, m.dim)})
             else:
-                e = {"state": (m.heads, m.vdim, m.dim)}
-                if m.conv > 1:
-                    e["tails"] = (m.conv - 1, 2 * m.kv_heads * m.dim + m.heads * m.vdim)
-                spec.append(e)
+                spec.append({"state": (m.heads, m.vdim, m.dim),
+                             "tails": (m.conv - 1, 2 * m.kv_heads * m.dim + m.heads * m.vdim)})
         return spec
 
     def make_cache(self, num_blocks: int, block_size: int, state_slots: int):

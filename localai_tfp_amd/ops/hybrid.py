@@ -419,8 +419,8 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     """Causal attention of q [T, H*dk] over the paged pools (rope_norm_append's layout); query head h reads key
     head g = h // (H / G) and value head g % v_heads (v_heads = G when not given; fewer value heads than key heads:
     several attention maps over the same values). `p32`: softmax weights enter the value product with more than
-    bf16's mantissa also in bf16 mode (the row kernels always do; the matrix-core kernels are left out, the GEMM
-    route splits each weight into two bf16 numbers). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
+    bf16's mantissa also in bf16 mode (the row kernels keep them in fp32 anyway; the matrix-core kernels and the GEMM
+    route split each weight into two bf16 numbers, its rounding and the rounding of the rest). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
     max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
     [H] adds exp(sink[h]). `bias` (fp32 [H, L], contiguous) adds bias[h, min(i - j, L - 1)] to the scaled score.
     `gate` (fp32 [T, H], may be a column slice) multiplies head h's output of row t by sigmoid(gate[t, h]). out
@@ -474,7 +474,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     nb = bias.shape[1] if bias is not None else 0
     ldg = gate.stride(0) if gate is not None else 0
     extra = (N.ptr(sink_v), N.ptr(bias), nb)  # the gate pointer moves with the rows a launch serves
-    mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and not p32 and \
+    mfma_ok = q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and MFMA_MIN_ROWS > 0 and \
         bool(N.hybrid_kernels().mxh_attention_mfma_ok(dk, dv))
     if nd:
         vis = rag.dec_max_len
@@ -494,7 +494,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), rag.dec_lens.data_ptr(), nd, out.data_ptr(),
                     out.stride(0), _is16(out), H, G, dk, dv, float(scale), int(chunk), int(window), int(sink),
                     float(out_scale), parts, plen if parts > 1 else 0, N.ptr(ml), N.ptr(po), *extra, N.ptr(gate), ldg,
-                    Gv, st)
+                    Gv, int(p32), st)
         else:
             N.kcall("mxh_attention", q.data_ptr(), q.stride(0), _is16(q), kc.data_ptr(), vc.data_ptr(), bs,
                     rag.dec_bt.data_ptr(), rag.dec_bt.stride(0), None, rag.dec_lens.data_ptr(), nd, nd, 0,
@@ -525,7 +525,7 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
                     N.kcall("mxh_attention_mfma", qk.data_ptr(), qk.stride(0), kc.data_ptr(), vc.data_ptr(), bs,
                             rag.pf_bt[k].data_ptr(), rag.pf_ctx_host[k] - n, n, ok.data_ptr(), ok.stride(0), _is16(out),
                             H, G, dk, dv, float(scale), int(chunk), int(window), int(sink), float(out_scale), *extra,
-                            N.ptr(gk), ldg, Gv, st)
+                            N.ptr(gk), ldg, Gv, int(p32), st)
                 else:
                     _attn_gemm_chunk(qk, kc, vc, rag.pf_bt[k], rag.pf_ctx_host[k] - n, n, H, G, dk, dv, scale, chunk,
                                      window, sink, ok, out_scale, sink_v, bias, gk, Gv, p32)
