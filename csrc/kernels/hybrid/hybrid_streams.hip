@@ -39,12 +39,19 @@ MX_DEV float block_sum_any(float v, float* red) {
 }
 
 template <bool B16>
-__global__ __launch_bounds__(NT) void embed_pair_kernel(const void* table, const void* pair, int V, const int* tokens,
-                                                        const int* seq_state, const int* positions, int n_dec,
-                                                        const int* pf_cu, int n_pf, int* last, float scale, int mp,
-                                                        int mc, int buckets, float* out, int copies, int C) {
-    const int t = blockIdx.x;
+__global__ __launch_bounds__(1024) void embed_pair_kernel(const void* __restrict__ table, const void* __restrict__ pair,
+                                                          int V, const int* __restrict__ tokens,
+                                                          const int* __restrict__ seq_state,
+                                                          const int* __restrict__ positions, int n_dec,
+                                                          const int* __restrict__ pf_cu, int n_pf, int* last,
+                                                          float scale, int mp, int mc, int buckets,
+                                                          float* __restrict__ out, int copies, int C) {
+    const int t = blockIdx.x, nt = blockDim.x;
+    // what does not depend on the row's chunk is asked for at once: the token, its position, the token above, and
+    // (decode rows) the slot; the chunk search of prompt rows follows
     const int raw = tokens[t];
+    const int pos = pair ? positions[t] : 0;
+    const int above = pair && t > 0 ? tokens[t - 1] : 0;
     const int tok = (raw < 0 || raw >= V) ? 0 : raw;
     long prow = -1;
     if (pair) {
@@ -62,10 +69,10 @@ __global__ __launch_bounds__(NT) void embed_pair_kernel(const void* table, const
             end = n_dec + pf_cu[lo + 1] - 1;
         }
         const int slot = seq_state[s];
-        if (positions[t] == 0) {
+        if (pos == 0) {
             prow = buckets;
         } else {
-            const long prev = t == first ? (slot >= 0 ? last[slot] : 0) : tokens[t - 1];
+            const long prev = t == first ? (slot >= 0 ? last[slot] : 0) : above;
             const long hsh = (prev * mp + (long)raw * mc) % buckets;
             prow = hsh < 0 ? hsh + buckets : hsh;
         }
@@ -76,19 +83,20 @@ __global__ __launch_bounds__(NT) void embed_pair_kernel(const void* table, const
     }
     const long base = (long)tok * C;
     float* o = out + (long)t * copies * C;
-    for (int c = threadIdx.x; c < C; c += NT) {
+    for (int c = threadIdx.x; c < C; c += nt) {
         float v = ld_e<B16>(table, base + c) * scale;
         if (prow >= 0) v += ld_e<B16>(pair, prow * C + c);
         for (int k = 0; k < copies; ++k) o[(long)k * C + c] = v;
     }
 }
 
-constexpr int HS_RK = 8;  // columns per thread whose weighted sum stays in registers
+// columns per thread whose old values are requested together and whose weighted sum stays in registers
 template <int S>
 __global__ __launch_bounds__(1024) void hyper_step_kernel(float* xs, const float* y, int ldy, const float* mix,
                                                           const float* ow, const float* iw, const float* nw,
                                                           float offset, float eps, float* h32, int ld32, bf16_t* h16,
                                                           int ld16, float* total, int ldt, int C) {
+    constexpr int HS_RK = S <= 2 ? 8 : 4;
     __shared__ float red[16];
     const int t = blockIdx.x, nt = blockDim.x;
     float* xr = xs + (long)t * S * C;
@@ -101,14 +109,12 @@ __global__ __launch_bounds__(1024) void hyper_step_kernel(float* xs, const float
 #pragma unroll
         for (int b = 0; b < S; ++b) m[a][b] = y ? mix[a * S + b] : (a == b ? 1.f : 0.f);
     }
-    // one column: the streams' update (stored), their sum (stored when asked for), and the next input's weighted sum
-    auto column = [&](int c) -> float {
-        float x[S], nx[S];
-#pragma unroll
-        for (int a = 0; a < S; ++a) x[a] = xr[(long)a * C + c];
+    // one column from its old values: the streams' update (stored), their sum (stored when asked for), and the next
+    // input's weighted sum
+    auto column = [&](int c, const float (&x)[S], float yv) -> float {
+        float nx[S];
         float u = 0.f, sum = 0.f;
         if (yr) {
-            const float yv = yr[c];
 #pragma unroll
             for (int b = 0; b < S; ++b) {
                 float v = 0.f;
@@ -129,16 +135,28 @@ __global__ __launch_bounds__(1024) void hyper_step_kernel(float* xs, const float
         if (total) total[(long)t * ldt + c] = sum;
         return u;
     };
-    float u[HS_RK];
+    // the stores of one column may not pass the loads of the next (the compiler sees the same array): the loads of
+    // all register columns go first, clamped and without branches, so that they are in flight together
+    float xo[HS_RK][S], yo[HS_RK], u[HS_RK];
+#pragma unroll
+    for (int k = 0; k < HS_RK; ++k) {
+        const int cc = min((int)threadIdx.x + k * nt, C - 1);
+#pragma unroll
+        for (int a = 0; a < S; ++a) xo[k][a] = xr[(long)a * C + cc];
+        yo[k] = yr ? yr[cc] : 0.f;
+    }
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < HS_RK; ++k) {
         const int c = threadIdx.x + k * nt;
-        u[k] = c < C ? column(c) : 0.f;
+        u[k] = c < C ? column(c, xo[k], yo[k]) : 0.f;
         ss += u[k] * u[k];
     }
     for (int c = threadIdx.x + HS_RK * nt; c < C; c += nt) {
-        const float v = column(c);
+        float x[S];
+#pragma unroll
+        for (int a = 0; a < S; ++a) x[a] = xr[(long)a * C + c];
+        const float v = column(c, x, yr ? yr[c] : 0.f);
         ss += v * v;
     }
     if (!iw) return;
@@ -159,6 +177,58 @@ __global__ __launch_bounds__(1024) void hyper_step_kernel(float* xs, const float
 #pragma unroll
         for (int b = 0; b < S; ++b) v += wi[b] * xr[(long)b * C + c];
         emit(c, v);
+    }
+}
+
+// More than 8 streams (up to 32): the same pass with the coefficients and a column's old values in LDS instead of
+// registers, one column at a time per thread; the next input is recomputed from the streams just written.
+__global__ __launch_bounds__(NT) void hyper_step_any_kernel(float* xs, const float* y, int ldy, const float* mix,
+                                                            const float* ow, const float* iw, const float* nw,
+                                                            float offset, float eps, float* h32, int ld32, bf16_t* h16,
+                                                            int ld16, float* total, int ldt, int S, int C) {
+    extern __shared__ float sm[];  // mix [S][S], out [S], in [S], old values [S][NT]
+    __shared__ float red[16];
+    float* cm = sm;
+    float* co = cm + S * S;
+    float* ci = co + S;
+    float* old = ci + S;
+    const int t = blockIdx.x, tid = threadIdx.x;
+    float* xr = xs + (long)t * S * C;
+    const float* yr = y ? y + (long)t * ldy : nullptr;
+    for (int i = tid; i < S * S; i += NT) cm[i] = y ? mix[i] : 0.f;
+    for (int i = tid; i < S; i += NT) {
+        co[i] = y ? ow[i] : 0.f;
+        ci[i] = iw ? iw[i] : 0.f;
+    }
+    __syncthreads();
+    float ss = 0.f;
+    for (int c = tid; c < C; c += NT) {
+        for (int a = 0; a < S; ++a) old[a * NT + tid] = xr[(long)a * C + c];
+        const float yv = yr ? yr[c] : 0.f;
+        float u = 0.f, sum = 0.f;
+        for (int b = 0; b < S; ++b) {
+            float v = old[b * NT + tid];
+            if (yr) {
+                v = 0.f;
+                for (int a = 0; a < S; ++a) v += cm[a * S + b] * old[a * NT + tid];
+                v += co[b] * yv;
+                xr[(long)b * C + c] = v;
+            }
+            u += ci[b] * v;
+            sum += v;
+        }
+        if (total) total[(long)t * ldt + c] = sum;
+        ss += u * u;
+    }
+    if (!iw) return;
+    ss = block_sum_any(ss, red);
+    const float sc = 1.f / sqrtf(ss / (float)C + eps);
+    for (int c = tid; c < C; c += NT) {  // the streams this thread has just written
+        float v = 0.f;
+        for (int b = 0; b < S; ++b) v += ci[b] * xr[(long)b * C + c];
+        v = v * sc * (offset + nw[c]);
+        if (h32) h32[(long)t * ld32 + c] = v;
+        if (h16) h16[(long)t * ld16 + c] = f32_to_bf16(v);
     }
 }
 
@@ -205,23 +275,27 @@ __global__ __launch_bounds__(64) void rope_rows_kernel(float* x, int ldx, const 
 
 // grid (T, C / group)
 template <bool B16>
-__global__ __launch_bounds__(NT) void diff_group_norm_kernel(const float* a, int lda, const float* b, int ldb, float lam,
+__global__ __launch_bounds__(256) void diff_group_norm_kernel(const float* a, int lda, const float* b, int ldb, float lam,
                                                              float eps, int group, float out_scale, void* out,
                                                              int ldo) {
     __shared__ float red[16];
-    const int t = blockIdx.x, c0 = blockIdx.y * group;
+    const int t = blockIdx.x, c0 = blockIdx.y * group, nt = blockDim.x;
     const float* ar = a + (long)t * lda + c0;
     const float* br = b + (long)t * ldb + c0;
-    constexpr int GC = 4;  // groups of up to NT * GC numbers stay in registers
+    constexpr int GC = 4;  // groups of up to blockDim * GC numbers stay in registers
     float z[GC];
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < GC; ++k) {
-        const int e = threadIdx.x + k * NT;
-        z[k] = e < group ? ar[e] - lam * br[e] : 0.f;
+        const int e = min((int)threadIdx.x + k * nt, group - 1);  // (clamped: both loads of all GC without a branch)
+        z[k] = ar[e] - lam * br[e];
+    }
+#pragma unroll
+    for (int k = 0; k < GC; ++k) {
+        if ((int)threadIdx.x + k * nt >= group) z[k] = 0.f;
         ss += z[k] * z[k];
     }
-    for (int e = threadIdx.x + GC * NT; e < group; e += NT) {
+    for (int e = threadIdx.x + GC * nt; e < group; e += nt) {
         const float v = ar[e] - lam * br[e];
         ss += v * v;
     }
@@ -233,10 +307,10 @@ __global__ __launch_bounds__(NT) void diff_group_norm_kernel(const float* a, int
     };
 #pragma unroll
     for (int k = 0; k < GC; ++k) {
-        const int e = threadIdx.x + k * NT;
+        const int e = threadIdx.x + k * nt;
         if (e < group) put(e, z[k]);
     }
-    for (int e = threadIdx.x + GC * NT; e < group; e += NT) put(e, ar[e] - lam * br[e]);
+    for (int e = threadIdx.x + GC * nt; e < group; e += nt) put(e, ar[e] - lam * br[e]);
 }
 
 }  // namespace
@@ -251,12 +325,13 @@ extern "C" int mxh_embed_pair(const void* table, const void* pair, int is16, int
     if (T <= 0) return 0;
     MXH_CHECK(table && tokens && out && V > 0 && C > 0 && copies >= 1 && n_dec >= 0 && n_dec <= T);
     MXH_CHECK(!pair || (seq_state && positions && last && buckets > 0 && (n_dec == T || (pf_cu && n_pf > 0))));
+    const int threads = C <= 1024 ? 256 : 1024;
     if (is16)
-        embed_pair_kernel<true><<<T, NT, 0, st>>>(table, pair, V, tokens, seq_state, positions, n_dec, pf_cu, n_pf, last,
-                                                  scale, mul_prev, mul_cur, buckets, out, copies, C);
+        embed_pair_kernel<true><<<T, threads, 0, st>>>(table, pair, V, tokens, seq_state, positions, n_dec, pf_cu, n_pf,
+                                                       last, scale, mul_prev, mul_cur, buckets, out, copies, C);
     else
-        embed_pair_kernel<false><<<T, NT, 0, st>>>(table, pair, V, tokens, seq_state, positions, n_dec, pf_cu, n_pf, last,
-                                                   scale, mul_prev, mul_cur, buckets, out, copies, C);
+        embed_pair_kernel<false><<<T, threads, 0, st>>>(table, pair, V, tokens, seq_state, positions, n_dec, pf_cu, n_pf,
+                                                        last, scale, mul_prev, mul_cur, buckets, out, copies, C);
     return (int)hipGetLastError();
 }
 
@@ -264,10 +339,16 @@ extern "C" int mxh_hyper_step(float* xs, const float* y, int ldy, const float* m
                               const float* nw, float offset, float eps, float* h32, int ld32, void* h16, int ld16,
                               float* total, int ldt, int T, int S, int C, hipStream_t st) {
     if (T <= 0) return 0;
-    MXH_CHECK(xs && S >= 1 && S <= 8 && C > 0);
+    MXH_CHECK(xs && S >= 1 && S <= 32 && C > 0);
     MXH_CHECK((!y || (mix && ow && ldy >= C)) && (!iw || (nw && (h32 || h16))) && (!h32 || ld32 >= C) &&
               (!h16 || ld16 >= C) && (!total || ldt >= C));
-    const int threads = C <= 2048 ? 256 : 1024;
+    if (S > 8) {
+        const size_t dyn = (size_t)(S * S + 2 * S + S * NT) * sizeof(float);
+        hyper_step_any_kernel<<<T, NT, dyn, st>>>(xs, y, ldy, mix, ow, iw, nw, offset, eps, h32, ld32, (bf16_t*)h16, ld16,
+                                                  total, ldt, S, C);
+        return (int)hipGetLastError();
+    }
+    const int threads = C <= 1024 ? 256 : 1024;
 #define GO(S_)                                                                                                        \
     case S_:                                                                                                          \
         hyper_step_kernel<S_><<<T, threads, 0, st>>>(xs, y, ldy, mix, ow, iw, nw, offset, eps, h32, ld32, (bf16_t*)h16, \
@@ -301,7 +382,8 @@ extern "C" int mxh_diff_group_norm(const float* a, int lda, const float* b, int 
     if (T <= 0) return 0;
     MXH_CHECK(a && b && out && group > 0 && C % group == 0 && C / group <= 65535 && lda >= C && ldb >= C && ldo >= C);
     const dim3 grid(T, C / group);
-    if (o16) diff_group_norm_kernel<true><<<grid, NT, 0, st>>>(a, lda, b, ldb, lam, eps, group, out_scale, out, ldo);
-    else diff_group_norm_kernel<false><<<grid, NT, 0, st>>>(a, lda, b, ldb, lam, eps, group, out_scale, out, ldo);
+    const int threads = group <= 256 ? 64 : NT;  // one wave for a head of ordinary size
+    if (o16) diff_group_norm_kernel<true><<<grid, threads, 0, st>>>(a, lda, b, ldb, lam, eps, group, out_scale, out, ldo);
+    else diff_group_norm_kernel<false><<<grid, threads, 0, st>>>(a, lda, b, ldb, lam, eps, group, out_scale, out, ldo);
     return (int)hipGetLastError();
 }

@@ -155,7 +155,7 @@ def embed_pair(table: torch.Tensor, pair: torch.Tensor | None, tokens: torch.Ten
     return out
 
 
-HYPER_MAX_STREAMS = 8
+HYPER_MAX_STREAMS = 32  # (up to 8 streams keep a column's values and the coefficients in registers)
 
 
 def hyper_step(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, out_w: torch.Tensor | None,

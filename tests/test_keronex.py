@@ -117,7 +117,8 @@ def test_pair_embedding_carries_the_previous_token(dev):
 def test_stream_update_read_and_sum(dev):
     g = torch.Generator().manual_seed(5)
     eps = 0.3  # a large eps shows whether it sits inside the root
-    for S, C, M in ((1, 40, 3), (3, 72, 5), (4, 2100, 2), (7, 300, 2), (8, 64, 2), (2, 9000, 2)):
+    for S, C, M in ((1, 40, 3), (3, 72, 5), (4, 2100, 2), (7, 300, 2), (8, 64, 2), (2, 9000, 2), (3, 5000, 2), (11, 300, 3),
+                    (32, 70, 2)):
         xs = torch.randn(M, S, C, generator=g) * 2
         y = torch.randn(M, C + 3, generator=g)
         mix, wo, wi = torch.randn(S, S, generator=g), torch.randn(S, generator=g), torch.randn(S, generator=g)
@@ -637,7 +638,7 @@ def test_config_reader_and_checkpoint_round_trip(tmp_path):
             L["mixer"].update(rank_a=L2.mixer.rank_a, rank_g=L2.mixer.rank_g)
     for path, val in ((("layers", 0, "type"), "something_else"), (("layers", 1, "mlp", "kind"), "glu"),
                       (("layers", 3, "weights_of"), 3), (("layers", 3, "weights_of"), 1), (("layers", 3, "mixer", "dim"), 8),
-                      (("layers", 2, "mixer", "decay"), [0.5]), (("streams",), 9), (("layers", 0, "mixer", "kv_heads"), 3)):
+                      (("layers", 2, "mixer", "decay"), [0.5]), (("streams",), 33), (("layers", 0, "mixer", "kv_heads"), 3)):
         bad = json.loads(json.dumps(j3))
         KE.KeronexConfig.from_json(bad)  # (valid until it is broken)
         node = bad
