@@ -260,7 +260,7 @@ def run_arch_bench(args) -> int:
                                 m_norm_groups=1, m_conv=4, name=f"vugotar-{sz}", **moe)
             yield "vugotar-moe", lambda: VU.VugotarModel.load(uc, VU.synthetic_source(uc, 1), dev, torch.bfloat16)
         elif args.arch_bench == "keronex":
-            # one differential-attention layer, two delta-rule layers with per-channel decays and a retention layer in
+            # two delta-rule layers with per-channel decays, one differential-attention layer and a retention layer in
             # turn, on four residual streams; attention heads as the Llama graph's (GQA 4:1) with two maps of 64 numbers
             # each over values of 128, half as many recurrent heads with 128 x 128 states; 8 experts of a quarter of the
             # feed-forward width, two chosen, and a shared expert of half of it. The closest model of the framework,
@@ -268,7 +268,7 @@ def run_arch_bench(args) -> int:
             # beside it with expert feed-forwards of the same widths.
             from localai_tfp_amd.models import keronex as KE
             from localai_tfp_amd.models import vugotar as VU
-            kinds = ("attention", "channel_delta", "channel_delta", "retention")
+            kinds = ("channel_delta", "channel_delta", "attention", "retention")
             moe = dict(experts=8, top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 2)
             kc = KE.make_config(hidden=s["hidden"], vocab=V, pattern=tuple(kinds[i % 4] for i in range(nl)),
                                 heads=s["heads"], kv_heads=max(1, s["heads"] // 4), dim=64, vdim=128, rot_dims=64,

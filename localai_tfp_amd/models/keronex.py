@@ -248,11 +248,11 @@ class KeronexConfig:
         return d
 
 
-def make_config(hidden=256, vocab=512, pattern=("attention", "channel_delta", "retention"), heads=4, kv_heads=2, dim=32,
-                vdim=32, scale=None, diff=0.5, rot_dims=None, rot_base=10000.0, r_heads=4, r_dim=32, r_vdim=32,
+def make_config(hidden=128, vocab=320, pattern=("retention", "attention", "channel_delta"), heads=4, kv_heads=2, dim=32,
+                vdim=32, scale=None, diff=0.25, rot_dims=None, rot_base=10000.0, r_heads=4, r_dim=32, r_vdim=32,
                 decay=None, r_rot_dims=None, d_heads=4, d_kv_heads=4, d_dim=32, d_vdim=32, conv=4, rank_a=8, rank_g=8,
                 mlps=("dense", "moe"), ff=512, experts=4, top=2, expert_ff=128, shared_ff=128, weights_of=None,
-                streams=4, emb_scale=1.0, bigram=(61, 7, 3), eps=1e-6, name="keronex") -> KeronexConfig:
+                streams=3, emb_scale=1.0, bigram=(61, 7, 3), eps=1e-6, name="keronex") -> KeronexConfig:
     """A configuration whose i-th layer has mixer pattern[i] and feed-forward mlps[i % len(mlps)] ("dense" | "moe" |
     None); `weights_of` maps a layer index to the earlier layer whose tensors it runs."""
     layers = []
@@ -278,19 +278,20 @@ def make_config(hidden=256, vocab=512, pattern=("attention", "channel_delta", "r
                          bigram=tuple(bigram) if bigram else None, streams=streams)
 
 
-# sizes of the order of a 1B / 7B decoder (bench / synthetic checkpoints): one attention layer, two delta-rule layers
-# and a retention layer in turn
-_PAT = ("attention", "channel_delta", "channel_delta", "retention")
+# sizes of the order of a 1B / 7B decoder (bench / synthetic checkpoints): two delta-rule layers, an attention layer
+# and a retention layer in turn, on four streams
+_PAT = ("channel_delta", "channel_delta", "attention", "retention")
 SYNTHETIC = {
-    "keronex-tiny": dict(hidden=256, vocab=512, pattern=_PAT + ("retention",), weights_of={4: 3}),
+    "keronex-tiny": dict(hidden=192, vocab=384, pattern=("retention", "attention", "channel_delta", "retention"),
+                         weights_of={3: 0}, streams=2),
     "keronex-1b": dict(hidden=2048, vocab=32000, pattern=_PAT * 4, heads=16, kv_heads=4, dim=64, vdim=128, r_heads=16,
                        r_dim=128, r_vdim=128, d_heads=16, d_kv_heads=16, d_dim=128, d_vdim=128, rank_a=32, rank_g=32,
                        mlps=("dense", "moe", "moe", "moe"), ff=8192, experts=8, top=2, expert_ff=2048, shared_ff=4096,
-                       bigram=(65521, 1009, 31)),
+                       streams=4, bigram=(65521, 1009, 31)),
     "keronex-7b": dict(hidden=4096, vocab=32000, pattern=_PAT * 8, heads=32, kv_heads=8, dim=64, vdim=128, r_heads=32,
                        r_dim=128, r_vdim=128, d_heads=32, d_kv_heads=32, d_dim=128, d_vdim=128, rank_a=32, rank_g=32,
                        mlps=("dense", "moe", "moe", "moe"), ff=14336, experts=8, top=2, expert_ff=3584, shared_ff=7168,
-                       bigram=(65521, 1009, 31)),
+                       streams=4, bigram=(65521, 1009, 31)),
 }
 
 

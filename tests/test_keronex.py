@@ -503,7 +503,7 @@ def _random_shape(rng):
                 rank_a=rng.choice([1, 4, 16]), rank_g=rng.choice([1, 4, 16]), mlps=mlps, ff=rng.choice([48, 128]),
                 experts=experts, top=rng.randint(1, experts), expert_ff=rng.choice([16, 40]),
                 shared_ff=rng.choice([0, 32, 96]), streams=rng.choice([None, 1, 2, 4, 6]),
-                emb_scale=rng.choice([1.0, 8.0]), bigram=rng.choice([None, (31, 5, 3), (509, 127, 19)]),
+                emb_scale=rng.choice([1.0, 8.0]), bigram=rng.choice([None, (31, 5, 3), (499, 113, 19)]),
                 eps=rng.choice([1e-6, 1e-5]))
 
 
