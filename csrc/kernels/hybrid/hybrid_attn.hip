@@ -1,10 +1,10 @@
 // hybrid_attn.hip: causal softmax attention over paged key / value pools with a visible range that starts at a chunk
 // border, a window's edge or position 0, and an optional sink term in the denominator (ops/hybrid.py
 // masked_attention). Pools are token-major: keys [blocks, bs, G * dk], values [blocks, bs, G * dv], fp32 or bf16.
-// The value pool may hold fewer heads than the key pool (gv of them, a divisor of G): key head g then reads value
-// head g % gv, several attention maps over the same values. Every kernel also takes an AttnExtra: a learned sink score per head instead of 0, an additive bias looked up by the
-// distance between query and key (table [H, distances], the last entry serving every larger distance), and a gate per
-// row and head whose sigmoid multiplies the head's output.
+// The value pool may hold fewer heads than the key pool (gv of them, a divisor of G): key head g then reads value head
+// g % gv, several attention maps over the same values. Every kernel also takes an AttnExtra: a learned sink score per
+// head instead of 0, an additive bias looked up by the distance between query and key (table [H, distances], the last
+// entry serving every larger distance), and a gate per row and head whose sigmoid multiplies the head's output.
 //
 // attn_rows_kernel: one wave per (query row, query head). Keys are taken 64 at a time, one per lane: the lane forms
 // its key's whole score against the query (held in LDS as fp32, pre-multiplied by the scale), the wave updates the

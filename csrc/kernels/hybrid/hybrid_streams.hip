@@ -8,7 +8,8 @@
 // hyper_step_kernel<S>: one block per row of S streams [S][C]. With y: all streams at once from the old ones,
 // x_t <- sum_s mix[s][t] x_s + out[t] y. With in: u = sum_t in[t] x_t of the new streams, h = u / rms(u) * (offset + w)
 // as fp32 and / or bf16. Optionally the sum of the new streams. The row is read once: u stays in registers between the
-// statistics and the output (columns beyond the register budget are recomputed from the streams just written).
+// statistics and the output (columns beyond the register budget are recomputed from the streams just written). More
+// than 8 streams take hyper_step_any_kernel, which keeps coefficients and a column's old values in LDS.
 // rope_rows_kernel: rotary positions in place on fp32 heads, neighbouring pairs or the pairs (i, i + rot / 2).
 // diff_group_norm_kernel: unit-RMS norm over groups of columns of a - lam * b.
 //
@@ -90,12 +91,12 @@ __global__ __launch_bounds__(1024) void embed_pair_kernel(const void* __restrict
     }
 }
 
-// columns per thread whose old values are requested together and whose weighted sum stays in registers
 template <int S>
 __global__ __launch_bounds__(1024) void hyper_step_kernel(float* xs, const float* y, int ldy, const float* mix,
                                                           const float* ow, const float* iw, const float* nw,
                                                           float offset, float eps, float* h32, int ld32, bf16_t* h16,
                                                           int ld16, float* total, int ldt, int C) {
+    // columns per thread whose old values are requested together and whose weighted sum stays in registers
     constexpr int HS_RK = S <= 2 ? 8 : 4;
     __shared__ float red[16];
     const int t = blockIdx.x, nt = blockDim.x;

@@ -170,7 +170,8 @@ class KeronexConfig:
             m, src = e["mixer"], e.get("weights_of")
             j = i if src is None else int(src)
             if src is not None:
-                _need(0 <= j < i and layers[j].weights_of is None, f"layer {i}: weights_of names an earlier layer with tensors")
+                _need(0 <= j < i and layers[j].weights_of is None,
+                      f"layer {i}: weights_of names an earlier layer with tensors")
                 _need(e["type"] == layers[j].type, f"layer {i}: same mixer as layer {j}")
             if e["type"] == "attention":
                 mixer = DiffAttnCfg(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]),

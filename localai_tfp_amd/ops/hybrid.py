@@ -223,7 +223,8 @@ def rope_norm_append(q_in: torch.Tensor, k_in: torch.Tensor, v_in: torch.Tensor,
                      half: bool = False, v_heads: int | None = None):
     """q_in [T, H*dk], k_in [T, G*dk], v_in [T, Gv*dv] (Gv = v_heads, G when not given: the value pool may hold fewer
     heads than the key pool): fp32 column slices of one projection output. Pair (2i, 2i+1), or with `half` the pair
-    (i, i + rot_dims/2), of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with `norm` every query
+    (i, i + rot_dims/2), of a head's first rot_dims numbers turns by positions[t] * rot_base^(-2i / rot_dims); with
+    `norm` every query
     and key head is then divided by its root mean square (eps inside the root) and multiplied by q_weight / k_weight
     (fp32 [dk], shared by the heads) when given. `q_temp` = (coef, every) multiplies the query at position p by
     1 + coef * ln(floor((p + 1) / every) + 1). Queries go to q_out [T, H*dk] (fp32 or bf16), keys and values into the
@@ -420,8 +421,8 @@ def masked_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, rag: R
     head g = h // (H / G) and value head g % v_heads (v_heads = G when not given; fewer value heads than key heads:
     several attention maps over the same values). `p32`: softmax weights enter the value product with more than
     bf16's mantissa also in bf16 mode (the row kernels keep them in fp32 anyway; the matrix-core kernels and the GEMM
-    route split each weight into two bf16 numbers, its rounding and the rounding of the rest). The row at position i sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`,
-    max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
+    route split each weight into two bf16 numbers, its rounding and the rounding of the rest). The row at position i
+    sees j in [lo, i]: lo = (i // chunk) * chunk with `chunk`, max(0, i - window + 1) with `window`, else 0. `sink` = True adds exp(0) to the softmax denominator, an fp32 tensor
     [H] adds exp(sink[h]). `bias` (fp32 [H, L], contiguous) adds bias[h, min(i - j, L - 1)] to the scaled score.
     `gate` (fp32 [T, H], may be a column slice) multiplies head h's output of row t by sigmoid(gate[t, h]). out
     [T, H*dv] (may be a column slice; fp32 or bf16) receives out_scale times the result. q, pools and out share fp32
@@ -617,8 +618,8 @@ def channel_decay(z: torch.Tensor, bias: torch.Tensor | None, tau: float, out: t
                   proj: torch.Tensor | None = None, rate_log: torch.Tensor | None = None):
     """out = sigmoid(x)^(1 / tau), computed as exp(log_sigmoid(x) / tau): the per-channel decay of gated linear
     attention; or, with `rate_log` (fp32 [heads], C / heads channels per head, tau unused),
-    out = exp(-exp(rate_log[head]) * softplus(x)): a step size per channel under a learned rate per head. x = z + bias with z fp32 [T, C]; or, with `proj` (fp32 [R, C], contiguous), x = z proj + bias with z
-    fp32 [T, R]: the second half of a low-rank projection, done in fp32 inside the same kernel. z may be a column
+    out = exp(-exp(rate_log[head]) * softplus(x)): a step size per channel under a learned rate per head. x = z + bias
+    with z fp32 [T, C]; or, with `proj` (fp32 [R, C], contiguous), x = z proj + bias with z fp32 [T, R]: the second half of a low-rank projection, done in fp32 inside the same kernel. z may be a column
     slice; bias fp32 [C]; out fp32 [T, C] contiguous."""
     T, C = out.shape
     if T == 0:
@@ -657,8 +658,9 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
     k, q fp32 [T, G*Nk] (head h reads group h // (H / G)), v fp32 [T, H*P], decay / coef fp32 [T, H], out fp32
     [T, H*P]; all may be column slices. With `channel` the decay is fp32 [T, H*Nk], one number per head and key
     channel (row n of S is multiplied by decay[h, n]: gated linear attention, or with `delta` a delta rule with a decay
-    per key channel). A decay of shape [H] is one constant per head for every token (retention). coef = None means 1; with `coef_sigmoid` coef holds
-    pre-activations (a column slice of a projection's output) and the write strength is their sigmoid.
+    per key channel). A decay of shape [H] is one constant per head for every token (retention). coef = None means 1;
+    with `coef_sigmoid` coef holds pre-activations (a column slice of a projection's output) and the write strength is
+    their sigmoid.
     state fp32 [slots, H, P, Nk] (a column's Nk numbers are contiguous) is read at
     the sequence's slot unless its first row is at position 0 (then S starts at zero) and written back after its last
     row."""
@@ -677,7 +679,9 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
                 vt = v[t].float().reshape(H, P)
                 dt = decay if decay.dim() == 1 else decay[t]
                 S = S * (dt.reshape(H, Nk)[:, :, None] if channel else dt[:, None, None])
-                cf = (torch.sigmoid(coef[t].float()) if coef_sigmoid else coef[t])[:, None] if coef is not None else 1.0
+                cf = 1.0
+                if coef is not None:
+                    cf = (torch.sigmoid(coef[t].float()) if coef_sigmoid else coef[t])[:, None]
                 u = cf * ((vt - torch.einsum("hnp,hn->hp", S, kt)) if delta else vt)
                 S = S + kt[:, :, None] * u[:, None, :]
                 o = torch.einsum("hnp,hn->hp", S, qt)
@@ -696,7 +700,8 @@ def state_scan(k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, decay: torch.T
         raise ValueError("state_scan: one fp32 decay per head, or per head and key channel")
     N.kcall("mxh_state_scan", k.data_ptr(), k.stride(0), q.data_ptr(), q.stride(0), v.data_ptr(), v.stride(0),
             decay.data_ptr(), 0 if decay.dim() == 1 else 1, N.ptr(coef),
-            coef.stride(0) if coef is not None else 0, int(coef_sigmoid), N.ptr(skip), state.data_ptr(), rag.state.data_ptr(),
+            coef.stride(0) if coef is not None else 0, int(coef_sigmoid), N.ptr(skip), state.data_ptr(),
+            rag.state.data_ptr(),
             rag.positions.data_ptr(), rag.n_dec, N.ptr(rag.pf_cu), rag.n_pf, out.data_ptr(), out.stride(0), H, G, Nk,
             P, int(delta), int(channel), float(q_scale), N.stream_ptr())
     return out
